@@ -123,7 +123,7 @@ class CacheManager:
         self.state: Dict[int, Dict[str, torch.Tensor]] = {}
         for entry, spec in state_specs.items():
             self.state[entry] = {
-                name: torch.zeros((self.max_requests,) + tuple(shape), dtype=dt, device=device)
+                name: torch.zeros((self.max_requests,) + tuple(shape), dtype=dt or dtype, device=device)
                 for name, (shape, dt) in spec.items()}
 
     # ------------------------------------------------------------ accounting

@@ -5,10 +5,11 @@ from .registry import (register_architecture, unregister_architecture, get_archi
 from .qwen2 import Qwen2Config
 from .vivevik import VivevikConfig
 from .ruvalorn import RuvalornConfig
+from .minodra import MinodraConfig
 
 __all__ = [
     "ConfigError", "WeightError", "UnsupportedSizeError", "PartSpec", "BlockSpec",
     "ScheduleEntry", "StreamOffset", "ModelSpec", "register_architecture", "unregister_architecture",
     "get_architecture", "registered_architectures", "architecture_of", "read_config",
-    "Architecture", "Qwen2Config", "VivevikConfig", "RuvalornConfig",
+    "Architecture", "Qwen2Config", "VivevikConfig", "RuvalornConfig", "MinodraConfig",
 ]

@@ -1270,7 +1270,8 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
 // Grouped products: `members` matrices [N, K] of equal shape lie one below the other in the packed
 // W (every member whole strips of 16 rows: N % 16 == 0); tile t of bm rows of the product belongs
 // to member tile_member[t] (-1: empty, its block leaves at once); row m reads row rows_index[m]
-// of x (null: row m).  out has M rows (a multiple of bm).  Epilogues: SWIGLU and F32.
+// of x (null: row m).  out has M rows (a multiple of bm).  Epilogues: SWIGLU, F32, and STORE
+// (compute dtype; epilogue 6: through max(z, 0)^2 first).
 extern "C" int llmlab_linear_grouped(const void* x, const void* w, int epilogue, void* out, int M, int N, int K,
                                      int ldo, int n_out, const int* tile_member, const int* rows_index, int bm,
                                      int wide, hipStream_t stream) {
@@ -1279,7 +1280,10 @@ extern "C" int llmlab_linear_grouped(const void* x, const void* w, int epilogue,
   LLMLAB_REQUIRE((bm == 64 || bm == 128) && M % bm == 0, "linear_grouped: %d rows in tiles of %d", M, bm);
   if (g_force_tile == 129) wide = 0;
   if (g_force_tile == 131) wide = 1;
-  LLMLAB_REQUIRE(epilogue == EPI_SWIGLU || epilogue == EPI_F32, "linear_grouped: epilogue %d", epilogue);
+  const int act = epilogue == 6 ? 1 : 0;
+  if (act) epilogue = EPI_STORE;
+  LLMLAB_REQUIRE(epilogue == EPI_SWIGLU || epilogue == EPI_F32 || epilogue == EPI_STORE, "linear_grouped: epilogue %d",
+                 epilogue);
   if (epilogue == EPI_SWIGLU)
     LLMLAB_REQUIRE(N % 32 == 0 && n_out > 0 && 2 * ((n_out + 15) / 16 * 16) == N,
                    "linear_grouped(swiglu): %d weight rows do not interleave %d outputs", N, n_out);
@@ -1287,13 +1291,23 @@ extern "C" int llmlab_linear_grouped(const void* x, const void* w, int epilogue,
     LLMLAB_REQUIRE(n_out <= N && n_out > N - 16, "linear_grouped: n_out %d, N %d", n_out, N);
   LLMLAB_REQUIRE(ldo >= n_out && tile_member != nullptr, "linear_grouped: output stride or tile table");
   if (M == 0) return 0;
-  EpiArgs e{out, nullptr, 0, ldo, n_out, 0, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, 0,
+  EpiArgs e{out, nullptr, 0, ldo, n_out, 0, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, act,
             tile_member, rows_index, (size_t)(N / 16) * (size_t)((K + 31) / 32) * 512};
   const bf16_t* A = (const bf16_t*)x;
   const bf16_t* W = (const bf16_t*)w;
   // (the columns past n_out of an F32 product are the zero rows that pad a member to whole strips)
   const int cols = epilogue == EPI_SWIGLU ? N : n_out;
-  if (bm == 64) {
+  if (epilogue == EPI_STORE) {
+    if (bm == 64)
+      hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_STORE, true>), dim3((cols + 63) / 64, M / 64, 1), dim3(256),
+                         0, stream, A, W, e, M, cols, K);
+    else if (wide)
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI_STORE, true>), dim3((cols + 255) / 256, M / 128, 1),
+                         dim3(512), 0, stream, A, W, e, M, cols, K);
+    else
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI_STORE, true>), dim3((cols + 127) / 128, M / 128, 1),
+                         dim3(256), 0, stream, A, W, e, M, cols, K);
+  } else if (bm == 64) {
     dim3 grid((cols + 63) / 64, M / 64, 1);
     if (epilogue == EPI_SWIGLU)
       hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_SWIGLU, true>), grid, dim3(256), 0, stream, A, W, e, M,

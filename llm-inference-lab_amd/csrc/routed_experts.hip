@@ -13,7 +13,8 @@ constexpr int SELECT_MAX_OUTPUTS = 1024;     // router outputs a row's wave keep
 // One wave a row.  Everything in float32; ties go to the smaller index, as a scan in order does.
 __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                         int outputs, int groups, int keep, int top, float scale,
-                                                        int* __restrict__ chosen, float* __restrict__ weights) {
+                                                        int* __restrict__ chosen, float* __restrict__ weights,
+                                                        int sigmoid) {
   __shared__ float s_score[SELECT_MAX_OUTPUTS], s_choice[SELECT_MAX_OUTPUTS];
   __shared__ float s_group[SELECT_MAX_OUTPUTS];
   const int row = blockIdx.x, lane = threadIdx.x;
@@ -23,12 +24,12 @@ __global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict_
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
   float sum = 0.f;
   for (int e = lane; e < outputs; e += WAVE) {
-    const float p = expf(z[e] - m);
+    const float p = sigmoid ? 1.f / (1.f + expf(-z[e])) : expf(z[e] - m);
     s_score[e] = p;
     sum += p;
   }
   for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-  const float inv = 1.f / sum;
+  const float inv = sigmoid ? 1.f : 1.f / sum;          // (sigmoid: every output scores by itself)
   for (int e = lane; e < outputs; e += WAVE) {
     const float s = s_score[e] * inv;
     s_score[e] = s;
@@ -99,7 +100,7 @@ __device__ __forceinline__ void wave_sync() {
 __device__ __forceinline__ void select_row_by_wave(const float* __restrict__ logits, const float* __restrict__ correction,
                                                    int outputs, int groups, int keep, int top, float scale,
                                                    int* __restrict__ chosen, float* __restrict__ weights, int row,
-                                                   int lane, float* s_wave) {
+                                                   int lane, float* s_wave, int sigmoid) {
   const bool mine = lane < outputs;
   const float z = mine ? logits[(size_t)row * outputs + lane] : -INFINITY;
   wave_sync();                                 // (the row before is read out)
@@ -107,12 +108,12 @@ __device__ __forceinline__ void select_row_by_wave(const float* __restrict__ log
   wave_sync();
   float m = -INFINITY;
   for (int j = 0; j < outputs; ++j) m = fmaxf(m, s_wave[j]);
-  const float p = mine ? expf(z - m) : 0.f;
+  const float p = mine ? (sigmoid ? 1.f / (1.f + expf(-z)) : expf(z - m)) : 0.f;
   s_wave[WAVE + lane] = p;
   wave_sync();
   float sum = 0.f;
   for (int j = 0; j < outputs; ++j) sum += s_wave[WAVE + j];         // (in the order of the outputs, on every lane)
-  const float score = p * (1.f / sum);
+  const float score = sigmoid ? p : p * (1.f / sum);
   float choice = mine ? score + correction[lane] : -INFINITY;
   wave_sync();
   s_wave[lane] = choice;
@@ -149,14 +150,17 @@ __device__ __forceinline__ void select_row_by_wave(const float* __restrict__ log
 __global__ __launch_bounds__(64) void moe_select_wave_kernel(const float* __restrict__ logits,
                                                              const float* __restrict__ correction, int outputs, int groups,
                                                              int keep, int top, float scale, int* __restrict__ chosen,
-                                                             float* __restrict__ weights) {
+                                                             float* __restrict__ weights, int sigmoid) {
   __shared__ float s_wave[2 * WAVE];
   select_row_by_wave(logits, correction, outputs, groups, keep, top, scale, chosen, weights, blockIdx.x, threadIdx.x,
-                     s_wave);
+                     s_wave, sigmoid);
 }
 
+// scoring: 0 softmax over the outputs, 1 the sigmoid of each output by itself
 extern "C" int llmlab_moe_select(const float* logits, const float* correction, int rows, int outputs, int groups,
-                                 int keep, int top, float scale, int* chosen, float* weights, hipStream_t stream) {
+                                 int keep, int top, float scale, int* chosen, float* weights, int scoring,
+                                 hipStream_t stream) {
+  LLMLAB_REQUIRE(scoring == 0 || scoring == 1, "moe_select: scoring %d", scoring);
   LLMLAB_REQUIRE(rows >= 0 && outputs > 0 && outputs <= SELECT_MAX_OUTPUTS,
                  "moe_select: a router of 1 to %d outputs, got %d", SELECT_MAX_OUTPUTS, outputs);
   LLMLAB_REQUIRE(groups > 0 && outputs % groups == 0 && keep > 0 && keep <= groups && top > 0 &&
@@ -165,10 +169,10 @@ extern "C" int llmlab_moe_select(const float* logits, const float* correction, i
   if (rows == 0) return 0;
   if (outputs <= WAVE)
     hipLaunchKernelGGL(moe_select_wave_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, outputs, groups,
-                       keep, top, scale, chosen, weights);
+                       keep, top, scale, chosen, weights, scoring);
   else
     hipLaunchKernelGGL(moe_select_kernel, dim3(rows), dim3(64), 0, stream, logits, correction, outputs, groups, keep,
-                       top, scale, chosen, weights);
+                       top, scale, chosen, weights, scoring);
   LLMLAB_LAUNCH_CHECK("moe_select");
   return 0;
 }
@@ -298,12 +302,14 @@ __global__ __launch_bounds__(1024) void moe_select_plan_kernel(const float* __re
                                                                int groups, int keep, int top, float scale,
                                                                int* __restrict__ chosen, float* __restrict__ weights,
                                                                int experts, int bm, int capacity, int* __restrict__ place_of,
-                                                               int* __restrict__ place_row, int* __restrict__ tile_member) {
+                                                               int* __restrict__ place_row, int* __restrict__ tile_member,
+                                                               int sigmoid) {
   __shared__ int s_count[PLAN_MAX_EXPERTS], s_start[PLAN_MAX_EXPERTS];
   __shared__ float s_waves[16][2 * WAVE];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
   for (int row = wave; row < rows; row += waves)
-    select_row_by_wave(logits, correction, outputs, groups, keep, top, scale, chosen, weights, row, lane, s_waves[wave]);
+    select_row_by_wave(logits, correction, outputs, groups, keep, top, scale, chosen, weights, row, lane, s_waves[wave],
+                       sigmoid);
   __threadfence_block();
   __syncthreads();
   plan_by_block(chosen, rows * top, experts, bm, capacity, place_of, place_row, tile_member, top, s_count, s_start);
@@ -311,9 +317,11 @@ __global__ __launch_bounds__(1024) void moe_select_plan_kernel(const float* __re
 
 extern "C" int llmlab_moe_select_plan(const float* logits, const float* correction, int rows, int outputs, int groups,
                                       int keep, int top, float scale, int* chosen, float* weights, int experts, int bm,
-                                      int capacity, int* place_of, int* place_row, int* tile_member, hipStream_t stream) {
+                                      int capacity, int* place_of, int* place_row, int* tile_member, int scoring,
+                                      hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && outputs > 0 && outputs <= WAVE, "moe_select_plan: a router of 1 to 64 outputs, got %d",
                  outputs);
+  LLMLAB_REQUIRE(scoring == 0 || scoring == 1, "moe_select_plan: scoring %d", scoring);
   LLMLAB_REQUIRE(groups > 0 && outputs % groups == 0 && keep > 0 && keep <= groups && top > 0 &&
                      top <= keep * (outputs / groups),
                  "moe_select_plan: %d outputs in %d groups of which %d are kept, top %d", outputs, groups, keep, top);
@@ -323,7 +331,7 @@ extern "C" int llmlab_moe_select_plan(const float* logits, const float* correcti
                  rows * top, experts);
   if (rows == 0) return 0;
   hipLaunchKernelGGL(moe_select_plan_kernel, dim3(1), dim3(1024), 0, stream, logits, correction, rows, outputs, groups,
-                     keep, top, scale, chosen, weights, experts, bm, capacity, place_of, place_row, tile_member);
+                     keep, top, scale, chosen, weights, experts, bm, capacity, place_of, place_row, tile_member, scoring);
   LLMLAB_LAUNCH_CHECK("moe_select_plan");
   return 0;
 }

@@ -1,0 +1,222 @@
+// Operations on the float32 residual stream around the sublayers of a layer, for gfx950:
+//   embed_pairs     x[r] = norm(table[id] * scale + pairs[hash(previous id, id)])
+//   causal_conv     out_t = h_t + sum_j w[:, j] h_(t - taps + 1 + j) over the positions of a request
+//   gated_add       x += y * sigmoid(gate + bias)
+//   softcap         x = cap * tanh(x / cap)
+// What a request's earlier steps left (its last token, the last inputs of a convolution) lives in
+// per-request slots; a step's rows of one request are adjacent.
+#include "common.h"
+
+extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
+
+// ------------------------------------------------------------------ embedding with hashed pairs
+// One block a row.  The pair row of a sequence's first token is row `buckets`; else
+// (previous * mul_prev + id * mul_cur) mod buckets, previous being the row before within the
+// step or, for a request's first row of the step, previous_slot[slot].  The block of a
+// request's first row also stores the request's LAST token of the step there, after it has read
+// the old one (one thread does both, in that order; no other block touches the slot).
+template <typename T>
+__global__ __launch_bounds__(256) void embed_pairs_kernel(
+    const T* __restrict__ table, const T* __restrict__ pairs, const int* __restrict__ ids,
+    const int* __restrict__ positions, const int* __restrict__ row_req, const int* __restrict__ q_start,
+    const int* __restrict__ req_rows, int* __restrict__ previous_slot, float scale, int vocab, int buckets,
+    long long mul_prev, long long mul_cur, const void* __restrict__ norm_w, int norm_bf16, float eps,
+    float* __restrict__ out, int hidden) {
+  __shared__ float red[17];
+  __shared__ int s_pair;
+  const int r = blockIdx.x;
+  int id = ids[r];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  if (threadIdx.x == 0) {
+    int pair = -1;
+    if (buckets > 0) {
+      const int b = row_req[r], first = q_start[b];
+      long long before = -1;
+      if (r > first) {
+        before = ids[r - 1];
+      } else {
+        const int slot = req_rows[b];
+        before = previous_slot[slot];
+        previous_slot[slot] = ids[q_start[b + 1] - 1];
+      }
+      if (before < 0) before = 0;
+      pair = positions[r] == 0 ? buckets : (int)((before * mul_prev + (long long)id * mul_cur) % buckets);
+    }
+    s_pair = pair;
+  }
+  __syncthreads();
+  const int pair = s_pair;
+  const T* t = table + (size_t)id * hidden;
+  const T* p = pair >= 0 ? pairs + (size_t)pair * hidden : nullptr;
+  float* o = out + (size_t)r * hidden;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    float v = to_float(t[c]) * scale;
+    if (p) v += to_float(p[c]);
+    o[c] = v;
+    ss += v * v;
+  }
+  if (!norm_w) return;
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = o[c] * inv * load_vec(norm_w, norm_bf16, c);
+}
+
+extern "C" int llmlab_embed_pairs(const void* table, const void* pairs, int dtype, const int* ids, const int* positions,
+                                  const int* row_req, const int* q_start, const int* req_rows, int* previous_slot,
+                                  float scale, int vocab, int buckets, long long mul_prev, long long mul_cur,
+                                  const void* norm_w, int norm_dtype, float eps, float* out, int rows, int hidden,
+                                  hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && hidden > 0 && vocab > 0 && buckets >= 0, "embed_pairs: bad sizes rows=%d hidden=%d", rows,
+                 hidden);
+  LLMLAB_REQUIRE(buckets == 0 || (pairs && positions && row_req && q_start && req_rows && previous_slot),
+                 "embed_pairs: the pairs need their table, the step's description and the slots");
+  if (rows == 0) return 0;
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(embed_pairs_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)table,
+                       (const bf16_t*)pairs, ids, positions, row_req, q_start, req_rows, previous_slot, scale, vocab,
+                       buckets, mul_prev, mul_cur, norm_w, norm_dtype == DT_BF16, eps, out, hidden);
+  else
+    hipLaunchKernelGGL(embed_pairs_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)table,
+                       (const float*)pairs, ids, positions, row_req, q_start, req_rows, previous_slot, scale, vocab,
+                       buckets, mul_prev, mul_cur, norm_w, norm_dtype == DT_BF16, eps, out, hidden);
+  LLMLAB_LAUNCH_CHECK("embed_pairs");
+  return 0;
+}
+
+// ------------------------------------------------------------------ short causal convolution
+// One block a row; a thread a channel.  Row r of request b (rows first .. first + n - 1 of the
+// step) reads the rows r - back of the step while they belong to b, and state[slot][taps - 1 -
+// (back - (r - first))] for the positions before the step (zeros before the sequence's start:
+// a slot is zeroed when a request is admitted).  state: [slots, taps - 1, width].
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ h, const float* __restrict__ w, int taps,
+                                                          const T* __restrict__ state, const int* __restrict__ row_req,
+                                                          const int* __restrict__ q_start,
+                                                          const int* __restrict__ req_rows, T* __restrict__ out,
+                                                          int width) {
+  const int r = blockIdx.x;
+  const int b = row_req[r], first = q_start[b];
+  const int inside = r - first;                       // rows of this request before r in the step
+  const T* st = state ? state + (size_t)req_rows[b] * (taps - 1) * width : nullptr;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float own = to_float(h[(size_t)r * width + c]);
+    float acc = own;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      float v = 0.f;
+      if (back == 0) v = own;
+      else if (back <= inside) v = to_float(h[(size_t)(r - back) * width + c]);
+      else if (st) v = to_float(st[(size_t)(taps - 1 - (back - inside)) * width + c]);
+      acc = fmaf(w[(size_t)c * taps + j], v, acc);
+    }
+    out[(size_t)r * width + c] = from_float<T>(acc);
+  }
+}
+
+// The slots after the step: the last taps - 1 inputs of the request, from what the slot held and
+// the step's rows.  The block of a request's first row does it for the whole request; a thread
+// reads place n + s before it writes place s, in rising order, so nothing is read after it changed.
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_state_kernel(const T* __restrict__ h, int taps, T* __restrict__ state,
+                                                                const int* __restrict__ row_req,
+                                                                const int* __restrict__ q_start,
+                                                                const int* __restrict__ req_rows, int width) {
+  const int r = blockIdx.x;
+  const int b = row_req[r], first = q_start[b];
+  if (r != first) return;
+  const int n = q_start[b + 1] - first, keep = taps - 1;
+  T* st = state + (size_t)req_rows[b] * keep * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x)
+    for (int s = 0; s < keep; ++s) {
+      const int at = n + s;                    // place in [what the slot held | the step's rows]
+      st[(size_t)s * width + c] = at < keep ? st[(size_t)at * width + c] : h[(size_t)(first + at - keep) * width + c];
+    }
+}
+
+extern "C" int llmlab_causal_conv(const void* h, int dtype, const float* w, int taps, void* state, const int* row_req,
+                                  const int* q_start, const int* req_rows, void* out, int rows, int width,
+                                  hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && width > 0 && taps >= 1, "causal_conv: bad sizes rows=%d width=%d taps=%d", rows, width, taps);
+  LLMLAB_REQUIRE(row_req && q_start && (taps == 1 || state == nullptr || req_rows),
+                 "causal_conv: the step's description is missing");
+  if (rows == 0) return 0;
+  if (dtype == DT_BF16) {
+    hipLaunchKernelGGL(causal_conv_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)h, w, taps,
+                       (const bf16_t*)state, row_req, q_start, req_rows, (bf16_t*)out, width);
+    if (state && taps > 1)
+      hipLaunchKernelGGL(causal_conv_state_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)h, taps,
+                         (bf16_t*)state, row_req, q_start, req_rows, width);
+  } else {
+    hipLaunchKernelGGL(causal_conv_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)h, w, taps,
+                       (const float*)state, row_req, q_start, req_rows, (float*)out, width);
+    if (state && taps > 1)
+      hipLaunchKernelGGL(causal_conv_state_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)h, taps,
+                         (float*)state, row_req, q_start, req_rows, width);
+  }
+  LLMLAB_LAUNCH_CHECK("causal_conv");
+  return 0;
+}
+
+// ------------------------------------------------------------------ gated sum into the stream
+// x[r, c] += y[r, c] * sigmoid(gate[r, c or 0] + bias[c]); gate null: x += y.  All float32.
+__global__ void gated_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gate,
+                                 int gate_cols, const float* __restrict__ bias, int width, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = i / width;
+    const int c = (int)(i - r * width);
+    float v = y[i];
+    if (gate) {
+      float g = gate_cols == 1 ? gate[r] : gate[i];
+      if (bias) g += bias[c];
+      v = v / (1.f + __expf(-g));
+    }
+    x[i] += v;
+  }
+}
+
+__global__ void gated_add4_kernel(floatx4* __restrict__ x, const floatx4* __restrict__ y, const floatx4* __restrict__ gate,
+                                  const floatx4* __restrict__ bias, int width4, size_t n4) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
+    floatx4 g = gate[i];
+    if (bias) g += bias[i % width4];
+    const floatx4 v = y[i];
+    floatx4 o = x[i];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] += v[q] / (1.f + __expf(-g[q]));
+    x[i] = o;
+  }
+}
+
+extern "C" int llmlab_gated_add(float* x, const float* y, const float* gate, int gate_cols, const float* bias, int rows,
+                                int width, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && width > 0 && (gate == nullptr || gate_cols == 1 || gate_cols == width),
+                 "gated_add: a gate per number or one per row, got %d columns for a width of %d", gate_cols, width);
+  const size_t n = (size_t)rows * width;
+  if (n == 0) return 0;
+  const bool vec = gate && gate_cols == width && width % 4 == 0 &&
+                   (((uintptr_t)x | (uintptr_t)y | (uintptr_t)gate | (uintptr_t)bias) & 15) == 0;
+  const size_t work = vec ? n / 4 : n;
+  const int blocks = (int)((work + 255) / 256 < 65535 ? (work + 255) / 256 : 65535);
+  if (vec)
+    hipLaunchKernelGGL(gated_add4_kernel, dim3(blocks), dim3(256), 0, stream, (floatx4*)x, (const floatx4*)y,
+                       (const floatx4*)gate, (const floatx4*)bias, width / 4, n / 4);
+  else
+    hipLaunchKernelGGL(gated_add_kernel, dim3(blocks), dim3(256), 0, stream, x, y, gate, gate_cols, bias, width, n);
+  LLMLAB_LAUNCH_CHECK("gated_add");
+  return 0;
+}
+
+// ------------------------------------------------------------------ soft cap
+__global__ void softcap_kernel(float* __restrict__ x, float cap, float inv_cap, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    x[i] = cap * tanhf(x[i] * inv_cap);
+}
+
+extern "C" int llmlab_softcap(float* x, float cap, size_t n, hipStream_t stream) {
+  LLMLAB_REQUIRE(cap > 0.f, "softcap: the cap must be positive, got %g", (double)cap);
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  hipLaunchKernelGGL(softcap_kernel, dim3(blocks), dim3(256), 0, stream, x, cap, 1.0f / cap, n);
+  LLMLAB_LAUNCH_CHECK("softcap");
+  return 0;
+}

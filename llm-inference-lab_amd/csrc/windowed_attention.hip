@@ -88,6 +88,9 @@ extern "C" int llmlab_project_norm_write(const float* proj, int ld, int rows, in
   return 0;
 }
 
+static int g_force_plain = 0;      // tests and measurements: no matrix-core kernel
+extern "C" void llmlab_debug_windowed_attention_plain(int on) { g_force_plain = on; }
+
 // ------------------------------------------------------------------ attention
 // The query at position i of its request attends to the keys i - window < j <= i and to the
 // kept prefix j < min(keep_first, i + 1); window <= 0: every j <= i.  Scores, the running maximum, the denominator
@@ -523,8 +526,6 @@ __global__ __launch_bounds__(64) void sink_window_attention_merge_kernel(MfmaArg
   }
 }
 
-static int g_force_plain = 0;
-extern "C" void llmlab_debug_windowed_attention_plain(int on) { g_force_plain = on; }
 
 // Whether the matrix-core kernel takes these sizes at all.
 extern "C" int llmlab_sink_window_attention_has_mfma(int dtype, int D, int E, int page_size) {
@@ -624,5 +625,160 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
                        E, (const float*)k_cache, (const float*)v_cache, table, max_pages, page_size, positions,
                        row_req, window, keep_first, sink, scale, (float*)out, q_start, long_from);
   LLMLAB_LAUNCH_CHECK("sink_window_attention");
+  return 0;
+}
+
+// ------------------------------------------------------------------ latent form
+// Attention over ONE cached vector per token (kv heads = 1, D = E = the vector's laid-out width,
+// the value pages holding the same vector in the values' order): every query head brings its
+// query in the vector's coordinates and gets a weighted sum of the vectors back.  The two
+// kernels below are what lies around the attention kernels in that form.
+//
+// One block a row.  proj[r, :] holds float32 projections [q latent (q_laid) | cached latent
+// (latent) | gates]: the query's latent is divided by the root mean square over its first
+// q_rank numbers and multiplied by q_w; the cached latent likewise (kv_rank, c_w) and written to
+// the row's place in both page tensors; the gates are copied as they are.  Numbers behind q_rank
+// / kv_rank are padding (zero projections, zero weights).
+template <typename T>
+__global__ __launch_bounds__(256) void latent_norm_write_kernel(
+    const float* __restrict__ proj, int ld, int q_rank, int q_laid, int kv_rank, int latent, int gates, float eps,
+    const float* __restrict__ q_w, const float* __restrict__ c_w, T* __restrict__ cq_out, float* __restrict__ gate_out,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int page_size, const int* __restrict__ positions,
+    const int* __restrict__ row_req, const int* __restrict__ table, int max_pages) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const float* src = proj + (size_t)r * ld;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < q_rank; c += blockDim.x) s += src[c] * src[c];
+  const float inv_q = 1.0f / sqrtf(block_sum(s, red) / (float)q_rank + eps);
+  s = 0.f;
+  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x) s += src[q_laid + c] * src[q_laid + c];
+  const float inv_c = 1.0f / sqrtf(block_sum(s, red) / (float)kv_rank + eps);
+  for (int c = threadIdx.x; c < q_laid; c += blockDim.x)
+    cq_out[(size_t)r * q_laid + c] = from_float<T>(src[c] * inv_q * q_w[c]);
+  for (int c = threadIdx.x; c < gates; c += blockDim.x) gate_out[(size_t)r * gates + c] = src[q_laid + latent + c];
+  const int pos = positions[r];
+  const int page = table[(size_t)row_req[r] * max_pages + pos / page_size];
+  const int slot = pos % page_size;
+  const size_t base = (size_t)page * page_size * latent;
+  for (int c = threadIdx.x; c < latent; c += blockDim.x) {
+    const T v = from_float<T>(src[q_laid + c] * inv_c * c_w[c]);
+    k_cache[base + (size_t)slot * latent + c] = v;
+    v_cache[base + value_index(slot, c, latent)] = v;
+  }
+}
+
+extern "C" int llmlab_latent_norm_write(const float* proj, int ld, int rows, int q_rank, int q_laid, int kv_rank,
+                                        int latent, int gates, float eps, const float* q_w, const float* c_w,
+                                        void* cq_out, float* gate_out, void* k_cache, void* v_cache, int dtype,
+                                        int page_size, const int* positions, const int* row_req, const int* table,
+                                        int max_pages, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && q_rank > 0 && q_laid >= q_rank && kv_rank > 0 && latent >= kv_rank && gates >= 0 &&
+                     page_size > 0 && page_size % 4 == 0,
+                 "latent_norm_write: bad sizes rows=%d q=%d/%d kv=%d/%d gates=%d page=%d", rows, q_rank, q_laid, kv_rank,
+                 latent, gates, page_size);
+  LLMLAB_REQUIRE(ld >= q_laid + latent + gates, "latent_norm_write: rows of %d numbers do not hold %d", ld,
+                 q_laid + latent + gates);
+  LLMLAB_REQUIRE(q_w && c_w && cq_out && k_cache && v_cache && positions && row_req && table && (gates == 0 || gate_out),
+                 "latent_norm_write: a pointer is missing");
+  if (rows == 0) return 0;
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(latent_norm_write_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, proj, ld, q_rank, q_laid,
+                       kv_rank, latent, gates, eps, q_w, c_w, (bf16_t*)cq_out, gate_out, (bf16_t*)k_cache,
+                       (bf16_t*)v_cache, page_size, positions, row_req, table, max_pages);
+  else
+    hipLaunchKernelGGL(latent_norm_write_kernel<float>, dim3(rows), dim3(256), 0, stream, proj, ld, q_rank, q_laid,
+                       kv_rank, latent, gates, eps, q_w, c_w, (float*)cq_out, gate_out, (float*)k_cache, (float*)v_cache,
+                       page_size, positions, row_req, table, max_pages);
+  LLMLAB_LAUNCH_CHECK("latent_norm_write");
+  return 0;
+}
+
+// out[r, a, :] = w[a] x[r, a, :] for a stack of matrices w [heads, N, K] (row-major), x [rows,
+// heads * K], out [rows, heads * N]: every head's numbers through that head's own matrix (a
+// query into the cached vector's coordinates; a weighted sum of cached vectors to the head's
+// values).  Sums in float32.
+//
+// Plain kernel (any sizes, both dtypes): a block per (row, head), the head's K numbers in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void head_products_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                            T* __restrict__ out, int heads, int N, int K) {
+  extern __shared__ float xs[];
+  const int r = blockIdx.x, a = blockIdx.y;
+  const T* xr = x + ((size_t)r * heads + a) * K;
+  for (int k = threadIdx.x; k < K; k += blockDim.x) xs[k] = to_float(xr[k]);
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int n = wave; n < N; n += nw) {                 // a wave an output: its lanes share the row of w
+    const T* wr = w + ((size_t)a * N + n) * K;
+    float s = 0.f;
+    for (int k = lane; k < K; k += 64) s = fmaf(to_float(wr[k]), xs[k], s);
+    s = wave_sum(s);
+    if (lane == 0) out[((size_t)r * heads + a) * N + n] = from_float<T>(s);
+  }
+}
+
+// Matrix-core kernel (bfloat16, K a multiple of 32, N of 16): a wave takes 16 rows of one head
+// and up to HP_TILES tiles of 16 outputs; the product is taken transposed, C^T = W x^T, so that
+// a lane ends up with four consecutive outputs of one row (one 8-byte store).
+constexpr int HP_TILES = 4;
+
+__global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                 bf16_t* __restrict__ out, int rows, int heads, int N,
+                                                                 int K) {
+  const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4, wave = threadIdx.x >> 6;
+  const int r0 = blockIdx.x * 16, a = blockIdx.y;
+  const int n_first = (blockIdx.z * 4 + wave) * HP_TILES * 16;
+  if (n_first >= N) return;
+  const int r = r0 + c;
+  const bool row_ok = r < rows;
+  const bf16_t* xr = x + ((size_t)(row_ok ? r : rows - 1) * heads + a) * K + 8 * g4;
+  const bf16_t* wa = w + (size_t)a * N * K;
+  floatx4 acc[HP_TILES];
+  const bf16_t* wr[HP_TILES];
+#pragma unroll
+  for (int t = 0; t < HP_TILES; ++t) {
+    acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const int n = n_first + 16 * t + c;
+    wr[t] = wa + (size_t)(n < N ? n : N - 1) * K + 8 * g4;       // (a tile past N is computed and not stored)
+  }
+  for (int k = 0; k < K; k += 32) {
+    const bf16x8 xf = *(const bf16x8*)(xr + k);
+#pragma unroll
+    for (int t = 0; t < HP_TILES; ++t) {
+      const bf16x8 wf = *(const bf16x8*)(wr[t] + k);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[t], 0, 0, 0);
+    }
+  }
+  if (!row_ok) return;
+#pragma unroll
+  for (int t = 0; t < HP_TILES; ++t) {
+    const int n = n_first + 16 * t + 4 * g4;
+    if (n >= N) continue;
+    bf16x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (bf16_t)acc[t][i];
+    *(bf16x4*)(out + ((size_t)r * heads + a) * N + n) = o;
+  }
+}
+
+extern "C" int llmlab_head_products(const void* x, const void* w, void* out, int dtype, int rows, int heads, int N,
+                                    int K, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0 && K <= 12288,
+                 "head_products: bad sizes rows=%d heads=%d N=%d K=%d", rows, heads, N, K);
+  if (rows == 0) return 0;
+  if (dtype == DT_BF16 && !g_force_plain && K % 32 == 0 && N % 16 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0 &&
+      ((uintptr_t)out & 7) == 0) {
+    dim3 grid((rows + 15) / 16, heads, (N + 4 * HP_TILES * 16 - 1) / (4 * HP_TILES * 16));
+    hipLaunchKernelGGL(head_products_mfma_kernel, grid, dim3(256), 0, stream, (const bf16_t*)x, (const bf16_t*)w,
+                       (bf16_t*)out, rows, heads, N, K);
+  } else if (dtype == DT_BF16) {
+    hipLaunchKernelGGL(head_products_kernel<bf16_t>, dim3(rows, heads), dim3(256), K * sizeof(float), stream,
+                       (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)out, heads, N, K);
+  } else {
+    hipLaunchKernelGGL(head_products_kernel<float>, dim3(rows, heads), dim3(256), K * sizeof(float), stream,
+                       (const float*)x, (const float*)w, (float*)out, heads, N, K);
+  }
+  LLMLAB_LAUNCH_CHECK("head_products");
   return 0;
 }

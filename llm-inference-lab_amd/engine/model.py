@@ -176,16 +176,26 @@ class CausalLM:
                     view.group, view.slot, view.writes_cache = owner.group, owner.slot, False
             elif entry.cache_of is not None:
                 raise ValueError(f"schedule[{view.index}] names a cache but its mixer keeps none")
-            st = mixer.state_spec()
+            # (a block arrangement with state of its own lists it together with its mixer's)
+            block = self.blocks[entry.block]
+            st = block.state_spec()
             if st:
                 state_specs[view.index] = dict(st)
+        # an embedding that remembers something of a sequence between steps keeps it in slots too
+        st = self.embedding.state_spec() if hasattr(self.embedding, "state_spec") else None
+        if st:
+            state_specs[self.EMBEDDING_STATE] = dict(st)
         return groups, state_specs
+
+    EMBEDDING_STATE = -1       # the embedding's key among the state specs (runs count from 0)
 
     def attach_cache(self, cache: CacheManager) -> None:
         for view in self.entries:
             if view.group is not None:
                 view.cache = {name: t[view.slot] for name, t in cache.storage[view.group].items()}
             view.state = cache.state.get(view.index, {})
+        if hasattr(self.embedding, "attach_state"):
+            self.embedding.attach_state(cache.state.get(self.EMBEDDING_STATE, {}))
 
     # ---------------------------------------------------------------- forward
     def forward(self, ctx) -> Optional[torch.Tensor]:

@@ -2,7 +2,7 @@
 
 Kinds of library: ``core`` (embedding, norms, rotary + cache write, matrix
 products, sampling), ``attn_d<D>`` (attention for head size D; one per head
-size that a model needs), ``windowed_attention``, ``linear_attention`` and ``routed_experts`` (parts whose
+size that a model needs), ``windowed_attention``, ``linear_attention``, ``routed_experts`` and ``stream_ops`` (parts whose
 sizes are run-time arguments; built when a model names them); beside them ``measure`` (stream and matrix-instruction loops for
 the benchmark's measured peaks) and the plain C++ references of the same operations,
 built with the host compiler for the tests.  A library's file name carries a hash of its sources
@@ -143,13 +143,15 @@ def attention_library(head_dim: int, force: bool = False) -> str:
 
 # Parts with run-time sizes: one library each, whatever the sizes of the model.
 MIXER_SOURCES = {"windowed_attention": "windowed_attention.hip", "linear_attention": "linear_attention.hip",
-                 "routed_experts": "routed_experts.hip"}
+                 "routed_experts": "routed_experts.hip", "stream_ops": "stream_ops.hip"}
 
 
 def mixer_library(kind: str, force: bool = False) -> str:
     """``windowed_attention``: sliding window with a kept prefix and a sink term;
     ``linear_attention``: the gated recurrence with a matrix state per head; ``routed_experts``: a
-    feed-forward of many experts of which a row uses a few (choice, sorting, grouped products)."""
+    feed-forward of many experts of which a row uses a few (choice, sorting, grouped products);
+    ``stream_ops``: what lies around the sublayers of a layer (an embedding with hashed token pairs, a
+    short causal convolution with per-request state, a gated sum into the stream, a soft cap)."""
     return _compile(kind, (MIXER_SOURCES[kind],), (), force)
 
 
@@ -201,7 +203,7 @@ def reference_library(force: bool = False) -> str:
 def library(kind: str, parameter=None, force: bool = False) -> str:
     """The library a part names in ``kernel_libraries()``: ``("core", None)`` or
     ``("attention", head_dim)``, ``("windowed_attention", None)``, ``("linear_attention", None)``,
-    ``("routed_experts", None)``."""
+    ``("routed_experts", None)``, ``("stream_ops", None)``."""
     if kind == "core":
         return core_library(force)
     if kind == "attention":

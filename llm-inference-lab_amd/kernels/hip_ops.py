@@ -1061,6 +1061,25 @@ class HipOps:
                 lib.llmlab_sink_window_attention_has_mfma.restype = _c_int
                 lib.llmlab_debug_windowed_attention_plain.argtypes = [_c_int]
                 lib.llmlab_debug_windowed_attention_plain.restype = None
+                lib.llmlab_latent_norm_write.argtypes = [
+                    _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr,
+                    _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
+                lib.llmlab_latent_norm_write.restype = _c_int
+                lib.llmlab_head_products.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                                     _c_ptr]
+                lib.llmlab_head_products.restype = _c_int
+            elif kind == "stream_ops":
+                lib.llmlab_embed_pairs.argtypes = [
+                    _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_int, _c_int,
+                    ctypes.c_longlong, ctypes.c_longlong, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_int, _c_ptr]
+                lib.llmlab_embed_pairs.restype = _c_int
+                lib.llmlab_causal_conv.argtypes = [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                                   _c_ptr, _c_int, _c_int, _c_ptr]
+                lib.llmlab_causal_conv.restype = _c_int
+                lib.llmlab_gated_add.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]
+                lib.llmlab_gated_add.restype = _c_int
+                lib.llmlab_softcap.argtypes = [_c_ptr, _c_float, _c_size, _c_ptr]
+                lib.llmlab_softcap.restype = _c_int
             elif kind == "linear_attention":
                 lib.llmlab_gla_decay.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr,
                                                  _c_int, _c_ptr]
@@ -1076,7 +1095,7 @@ class HipOps:
                 lib.llmlab_gla_output.restype = _c_int
             elif kind == "routed_experts":
                 lib.llmlab_moe_select.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                                  _c_ptr, _c_ptr, _c_ptr]
+                                                  _c_ptr, _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_moe_select.restype = _c_int
                 lib.llmlab_moe_add_chosen.argtypes = [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
                                                       _c_int, _c_int, _c_ptr]
@@ -1086,7 +1105,7 @@ class HipOps:
                 lib.llmlab_moe_plan.restype = _c_int
                 lib.llmlab_moe_select_plan.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                                                        _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                                                       _c_ptr]
+                                                       _c_int, _c_ptr]
                 lib.llmlab_moe_select_plan.restype = _c_int
                 lib.llmlab_moe_combine.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                                                    _c_int, _c_int, _c_ptr]
@@ -1140,8 +1159,10 @@ class HipOps:
         """Whether choice and sorting of a step of so many rows are one launch (``moe_select_plan``)."""
         return 0 < rows <= self.rules.select_plan_max_rows and outputs <= 64
 
+    SCORINGS = {"softmax": 0, "sigmoid": 1}
+
     def moe_select_plan(self, logits, correction, groups: int, groups_keep: int, scale: float, chosen, weights,
-                        num_experts: int, scratch) -> "MoePlan":
+                        num_experts: int, scratch, scoring: str = "softmax") -> "MoePlan":
         """``moe_select`` and ``moe_plan`` in one launch of one block, for steps of few rows."""
         lib = self._mixer_lib("routed_experts")
         for t, name, dt in ((logits, "router logits", torch.float32), (correction, "router correction", torch.float32),
@@ -1156,7 +1177,7 @@ class HipOps:
         self._call(lib.llmlab_moe_select_plan, self._ptr(logits), self._ptr(correction), rows, outputs, int(groups),
                    int(groups_keep), top, float(scale), self._ptr(chosen), self._ptr(weights), int(num_experts), plan.bm,
                    plan.capacity, self._ptr(plan.place_of), self._ptr(plan.place_row), self._ptr(plan.tile_member),
-                   self._stream(), lib=lib)
+                   self.SCORINGS[scoring], self._stream(), lib=lib)
         return plan
 
     def moe_plan(self, chosen, num_experts: int, scratch) -> "MoePlan":
@@ -1197,6 +1218,13 @@ class HipOps:
             raise ValueError("moe_gate_up: the experts' gate and up rows do not interleave the outputs")
         self._grouped(h, w_gate_up, plan, act, EPI_SWIGLU, act.shape[1], plan.place_row)
 
+    def moe_up_relu2(self, h, w_up: "StackedWeight", plan: "MoePlan", act) -> None:
+        """``act[place] = max(h[row] Wu_e^T, 0) ** 2`` for every place of the plan (experts without a
+        gate matrix); the square is taken on the float32 sums."""
+        if act.dtype != torch.bfloat16 or act.shape[1] != w_up.padded:
+            raise ValueError("moe_up_relu2: one output per (padded) row of an expert's up matrix")
+        self._grouped(h, w_up, plan, act, EPI_RELU2, act.shape[1], plan.place_row)
+
     def moe_down(self, act, w_down: "StackedWeight", plan: "MoePlan", y) -> None:
         """``y[place] = act[place] Wd_e^T`` in float32."""
         if y.dtype != torch.float32 or y.shape[1] != w_down.n:
@@ -1218,8 +1246,10 @@ class HipOps:
                    self._ptr(plan.place_of), self._ptr(chosen), self._ptr(weights), rows, chosen.shape[1],
                    int(num_experts), hidden, self._stream(), lib=lib)
 
-    def moe_select(self, logits, correction, groups: int, groups_keep: int, scale: float, chosen, weights) -> None:
-        """Per row of the router's float32 ``logits [rows, outputs]``: scores ``softmax(logits)``; choice
+    def moe_select(self, logits, correction, groups: int, groups_keep: int, scale: float, chosen, weights,
+                   scoring: str = "softmax") -> None:
+        """Per row of the router's float32 ``logits [rows, outputs]``: scores ``softmax(logits)``
+        (``scoring="sigmoid"``: the sigmoid of every logit by itself); choice
         values ``score + correction``; the outputs form ``groups`` equal groups of neighbours of which
         the ``groups_keep`` with the largest best choice value stay; ``chosen [rows, top]`` (int32) are
         the outputs with the largest choice values among those (ties: the smaller index), ``weights
@@ -1234,7 +1264,8 @@ class HipOps:
         if correction.numel() != outputs or tuple(chosen.shape) != (rows, top) or tuple(weights.shape) != (rows, top):
             raise ValueError("moe_select: shapes do not fit")
         self._call(lib.llmlab_moe_select, self._ptr(logits), self._ptr(correction), rows, outputs, int(groups),
-                   int(groups_keep), top, float(scale), self._ptr(chosen), self._ptr(weights), self._stream(), lib=lib)
+                   int(groups_keep), top, float(scale), self._ptr(chosen), self._ptr(weights), self.SCORINGS[scoring],
+                   self._stream(), lib=lib)
 
     def moe_add_chosen(self, resid, src, chosen, weights, first: int, last: int) -> None:
         """``resid[r] += w_r * src[r]`` with ``w_r`` the sum of ``weights[r, k]`` over the ``k`` whose
@@ -1459,6 +1490,145 @@ class HipOps:
                    self._stream(), lib=lib)
 
     # --------------------------------------------------------------- sampling
+    # ------------------------------ the stream around sublayers; the latent form of attention
+    def embed_pairs(self, table, pairs, ids, positions, row_req, q_start, req_rows, previous, scale: float,
+                    buckets: int, mul_prev: int, mul_cur: int, norm_weight, eps: float, out) -> None:
+        """``out[r] = norm(table[id_r] * scale + pairs[row_r])`` into the float32 stream.  ``row_r`` is
+        ``buckets`` for a sequence's first token, else ``(previous id * mul_prev + id * mul_cur) mod
+        buckets``; the id before a request's first row of the step comes from ``previous [slots, 1]``
+        (int32), which then takes the request's last id of the step.  ``norm_weight``: the weight of an
+        RMS norm over the sum (None: no norm).  ``buckets`` 0: no pairs."""
+        lib = self._mixer_lib("stream_ops")
+        self._need(table, "embedding table")
+        self._need(out, "residual stream", torch.float32)
+        self._need(ids, "token ids", torch.int32)
+        rows, hidden = out.shape
+        if table.dim() != 2 or table.shape[1] != hidden or ids.numel() < rows:
+            raise ValueError(f"embed_pairs: table {tuple(table.shape)}, {ids.numel()} ids, stream {tuple(out.shape)}")
+        if buckets:
+            self._need(pairs, "pair table", table.dtype)
+            self._need(previous, "previous-token slots", torch.int32)
+            if tuple(pairs.shape) != (buckets + 1, hidden):
+                raise ValueError(f"embed_pairs: a pair table of {buckets} buckets and one more row, got {tuple(pairs.shape)}")
+            for t, name, least in ((positions, "positions", rows), (row_req, "row -> request map", rows),
+                                   (q_start, "request row starts", 2), (req_rows, "request slots", 1)):
+                self._need(t, name, torch.int32)
+                if t.numel() < least:
+                    raise ValueError(f"embed_pairs: {name} is too short")
+        if norm_weight is not None:
+            self._need(norm_weight, "norm weight")
+            if norm_weight.numel() != hidden:
+                raise ValueError("embed_pairs: the norm's weight spans the stream's width")
+        self._call(lib.llmlab_embed_pairs, self._ptr(table), self._ptr(pairs) if buckets else None, _dt(table),
+                   self._ptr(ids), self._ptr(positions) if buckets else None, self._ptr(row_req) if buckets else None,
+                   self._ptr(q_start) if buckets else None, self._ptr(req_rows) if buckets else None,
+                   self._ptr(previous) if buckets else None, float(scale), table.shape[0], int(buckets), int(mul_prev),
+                   int(mul_cur), self._ptr(norm_weight), _dt(norm_weight) if norm_weight is not None else DT_F32,
+                   float(eps), self._ptr(out), rows, hidden, self._stream(), lib=lib)
+
+    def causal_conv(self, h, weight, state, positions, row_req, q_start, req_rows, out) -> None:
+        """``out_t = h_t + sum_j weight[:, j] h_(t - taps + 1 + j)`` channel by channel over the positions
+        of each request (``weight [width, taps]`` float32).  Inputs from before the step are read
+        from ``state [slots, taps - 1, width]`` (the latest last; zeros before a sequence's start),
+        which then takes each request's latest inputs.  ``h``, ``out``, ``state``: one kernel dtype."""
+        lib = self._mixer_lib("stream_ops")
+        self._need(h, "convolution input")
+        self._need(out, "convolution output", h.dtype)
+        self._need(weight, "convolution taps", torch.float32)
+        rows, width = h.shape
+        taps = weight.shape[1]
+        if tuple(weight.shape) != (width, taps) or tuple(out.shape) != (rows, width):
+            raise ValueError(f"causal_conv: input {tuple(h.shape)}, taps {tuple(weight.shape)}, output {tuple(out.shape)}")
+        if state is not None:
+            self._need(state, "convolution state", h.dtype)
+            if tuple(state.shape[1:]) != (taps - 1, width):
+                raise ValueError(f"causal_conv: state {tuple(state.shape)} does not hold {taps - 1} inputs of {width}")
+        elif taps > 1:
+            raise ValueError("causal_conv: more than one tap needs the slots of the requests")
+        for t, name, least in ((row_req, "row -> request map", rows), (q_start, "request row starts", 2),
+                               (req_rows, "request slots", 1)):
+            self._need(t, name, torch.int32)
+            if t.numel() < least:
+                raise ValueError(f"causal_conv: {name} is too short")
+        self._call(lib.llmlab_causal_conv, self._ptr(h), _dt(h), self._ptr(weight), taps, self._ptr(state),
+                   self._ptr(row_req), self._ptr(q_start), self._ptr(req_rows), self._ptr(out), rows, width,
+                   self._stream(), lib=lib)
+
+    def gated_add(self, x, y, gate, bias) -> None:
+        """``x += y * sigmoid(gate + bias)``, all float32: ``gate [rows, width]``, or ``[rows, 1]`` for
+        one number a row; ``bias [width]`` or None; ``gate`` None: ``x += y``."""
+        lib = self._mixer_lib("stream_ops")
+        self._need(x, "residual stream", torch.float32)
+        self._need(y, "sublayer output", torch.float32)
+        rows, width = x.shape
+        if tuple(y.shape) != (rows, width):
+            raise ValueError(f"gated_add: {tuple(y.shape)} onto {tuple(x.shape)}")
+        cols = 0
+        if gate is not None:
+            self._need(gate, "gate", torch.float32)
+            cols = gate.shape[1]
+            if gate.shape[0] != rows or cols not in (1, width):
+                raise ValueError(f"gated_add: gates {tuple(gate.shape)} for {tuple(x.shape)}")
+        if bias is not None:
+            self._need(bias, "gate bias", torch.float32)
+            if bias.numel() != width or gate is None:
+                raise ValueError("gated_add: a bias per column of a gate")
+        self._call(lib.llmlab_gated_add, self._ptr(x), self._ptr(y), self._ptr(gate), cols, self._ptr(bias), rows, width,
+                   self._stream(), lib=lib)
+
+    def softcap(self, x, cap: float) -> None:
+        """``x = cap * tanh(x / cap)`` in place, float32."""
+        lib = self._mixer_lib("stream_ops")
+        self._need(x, "logits", torch.float32)
+        self._call(lib.llmlab_softcap, self._ptr(x), float(cap), x.numel(), self._stream(), lib=lib)
+
+    def latent_norm_write(self, proj, q_rank: int, q_laid: int, kv_rank: int, latent: int, gates: int, q_norm, c_norm,
+                          eps: float, cq_out, gate_out, k_cache, v_cache, page_size: int, positions, row_req,
+                          block_table) -> None:
+        """From the float32 projections ``proj [rows, q_laid + latent + gates]``: the query's latent (RMS
+        norm over its first ``q_rank`` numbers, weight ``q_norm [q_laid]``) into ``cq_out [rows,
+        q_laid]``; the cached latent (RMS norm over ``kv_rank`` numbers, weight ``c_norm [latent]``)
+        into the row's place of both page tensors (``k``: row by row, ``v``: in quads of keys); the
+        gates as they are into ``gate_out [rows, gates]``."""
+        lib = self._mixer_lib("windowed_attention")
+        self._need(proj, "projections", torch.float32)
+        self._need(cq_out, "query latent")
+        rows = cq_out.shape[0]
+        if tuple(proj.shape) != (rows, q_laid + latent + gates) or tuple(cq_out.shape) != (rows, q_laid):
+            raise ValueError(f"latent_norm_write: projections {tuple(proj.shape)}, query latent {tuple(cq_out.shape)}")
+        self._need(q_norm, "query latent norm weight", torch.float32)
+        self._need(c_norm, "cached latent norm weight", torch.float32)
+        if q_norm.numel() != q_laid or c_norm.numel() != latent or not 0 < q_rank <= q_laid or not 0 < kv_rank <= latent:
+            raise ValueError("latent_norm_write: the norms' weights span the laid-out latents")
+        if gates:
+            self._need(gate_out, "head gates", torch.float32)
+            if tuple(gate_out.shape) != (rows, gates):
+                raise ValueError("latent_norm_write: one gate per row and head")
+        self._paged(k_cache, v_cache, 1, page_size, latent, latent, cq_out.dtype)
+        for t, name in ((positions, "positions"), (row_req, "row -> request map"), (block_table, "block table")):
+            self._need(t, name, torch.int32, contiguous=name != "block table")
+        if positions.numel() < rows or row_req.numel() < rows or block_table.stride(1) != 1:
+            raise ValueError("latent_norm_write: one position and one request index per row")
+        self._call(lib.llmlab_latent_norm_write, self._ptr(proj), proj.stride(0), rows, int(q_rank), int(q_laid),
+                   int(kv_rank), int(latent), int(gates), float(eps), self._ptr(q_norm), self._ptr(c_norm),
+                   self._ptr(cq_out), self._ptr(gate_out) if gates else None, self._ptr(k_cache), self._ptr(v_cache),
+                   _dt(cq_out), page_size, self._ptr(positions), self._ptr(row_req), self._ptr(block_table),
+                   block_table.stride(0), self._stream(), lib=lib)
+
+    def head_products(self, x, w, out) -> None:
+        """``out[r, a, :] = w[a] x[r, a, :]`` for a stack of matrices ``w [heads, n, k]``: ``x [rows, heads *
+        k]``, ``out [rows, heads * n]``, all of one kernel dtype; sums in float32."""
+        lib = self._mixer_lib("windowed_attention")
+        self._need(x, "head inputs")
+        self._need(w, "head matrices", x.dtype)
+        self._need(out, "head outputs", x.dtype)
+        heads, n, k = w.shape
+        rows = x.shape[0]
+        if tuple(x.shape) != (rows, heads * k) or tuple(out.shape) != (rows, heads * n):
+            raise ValueError(f"head_products: x {tuple(x.shape)}, matrices {tuple(w.shape)}, out {tuple(out.shape)}")
+        self._call(lib.llmlab_head_products, self._ptr(x), self._ptr(w), self._ptr(out), _dt(x), rows, heads, n, k,
+                   self._stream(), lib=lib)
+
     def argmax(self, logits, out, one_pass: bool = True) -> None:
         """``out[r]`` = the largest logit's index (the smallest among equals; -1 for a row
         without a finite value).  ``one_pass=False``: in two kernels, without the counters."""

@@ -5,6 +5,7 @@ from .norms import RMSNorm, LayerNorm
 from .positions import RotaryEmbedding, NoPosition
 from .attention import GQAAttention, WindowedSinkAttention
 from .linear_attention import GatedLinearAttention
+from .latent_attention import LatentAttention
 from .feed_forward import SwiGLU, DenseFeedForward, interleave_gate_up
 from .experts import RoutedExperts
-from .blocks import PreNormBlock, SublayerNormBlock, TokenEmbedding, LinearHead
+from .blocks import PreNormBlock, SublayerNormBlock, GatedConvBlock, TokenEmbedding, PairHashEmbedding, LinearHead

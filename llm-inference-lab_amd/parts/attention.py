@@ -272,6 +272,23 @@ class GQAAttention(Mixer):
         return total
 
 
+def rows_by_kernel(ops, ctx, dtype, key_dim, value_dim, page_size):
+    """``(long_from, launches)`` of this step for the attention kernels with run-time sizes: requests
+    of at least ``long_from`` rows go to the matrix-core kernel; worked out once per step, kept in
+    the step's notes for the other layers."""
+    pick = getattr(ops, "windowed_attention_long_rows", None)
+    long_from = pick(dtype, key_dim, value_dim, page_size) if pick is not None else 0
+    if not long_from:
+        return 0, 1
+    key = ("windowed_attention.split", long_from)
+    if key not in ctx.memo:
+        starts = ctx.host_q_start
+        counts = [starts[b + 1] - starts[b] for b in range(ctx.n_reqs)]
+        ctx.memo[key] = ((1 if any(n < long_from for n in counts) else 0)
+                         | (2 if any(n >= long_from for n in counts) else 0))
+    return long_from, ctx.memo[key]
+
+
 class WindowedSinkAttention(Mixer):
     """Grouped-query attention through a sliding window that keeps a sequence's first
     positions in sight, with a learned extra term in the softmax's denominator.
@@ -405,19 +422,7 @@ class WindowedSinkAttention(Mixer):
         self.ops.add_pending(residual, PendingSums(y, 1))
 
     def _split(self, ctx, page_size):
-        """``(long_from, launches)`` of this step: requests of at least ``long_from`` rows go to the
-        matrix-core kernel; worked out once per step, kept in the step's notes for the other layers."""
-        pick = getattr(self.ops, "windowed_attention_long_rows", None)
-        long_from = pick(self.dtype, self.key_dim, self.value_dim, page_size) if pick is not None else 0
-        if not long_from:
-            return 0, 1
-        key = ("windowed_attention.split", long_from)
-        if key not in ctx.memo:
-            starts = ctx.host_q_start
-            counts = [starts[b + 1] - starts[b] for b in range(ctx.n_reqs)]
-            ctx.memo[key] = ((1 if any(n < long_from for n in counts) else 0)
-                             | (2 if any(n >= long_from for n in counts) else 0))
-        return long_from, ctx.memo[key]
+        return rows_by_kernel(self.ops, ctx, self.dtype, self.key_dim, self.value_dim, page_size)
 
     keeps_launches = True      # (what depends on the step beyond its rows is asked for at the launch)
 

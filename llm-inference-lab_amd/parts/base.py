@@ -282,5 +282,11 @@ class Block(Part):
     def mixer_part(self) -> Mixer:
         raise NotImplementedError
 
+    def state_spec(self) -> Dict[str, Tuple[Tuple[int, ...], torch.dtype]]:
+        """Fixed-size per-request state of a run of this block: its mixer's, and whatever the
+        arrangement itself remembers of a sequence between steps (name -> (shape, dtype); a dtype
+        of None is the compute dtype).  All of it arrives in ``entry.state``."""
+        return self.mixer_part().state_spec()
+
     def forward(self, residual: torch.Tensor, ctx, entry) -> None:
         raise NotImplementedError

@@ -6,7 +6,7 @@ from typing import Dict
 import torch
 
 from ..config.spec import PartSpec
-from ..weights.loader import TensorSpec, MATRIX
+from ..weights.loader import TensorSpec, MATRIX, VECTOR, INIT_ZEROS
 from .base import Block, Part, NormedInput
 from .registry import register_part, build_part
 
@@ -149,6 +149,125 @@ class SublayerNormBlock(Block):
         return sum(p.weight_bytes() for p in self.parts())
 
 
+class GatedConvBlock(Block):
+    """A pre-norm layer whose sublayers read their input through a short causal convolution and
+    whose results pass a gate before they are summed::
+
+        h = norm1(x);  x += mixer(h + conv1(h)) * sigmoid(R1 h + b1)
+        h = norm2(x);  x += feed_forward(h + conv2(h)) * sigmoid(R2 h + b2)
+
+    ``conv(h)_t = sum_j w[:, j] * h_(t - taps + 1 + j)`` channel by channel over the positions of
+    one sequence (``w [width, taps]``, nothing before the sequence's start); the last ``taps - 1``
+    inputs of each convolution are per-request state, so a sequence may be cut anywhere.  The gate
+    reads the normed ``h`` itself, before the convolution (``R [width, width]``, ``b [width]``).
+    ``conv_taps=0``: no convolution; ``residual_gate=False``: the plain sum.  The stream, the
+    sigmoid and the sums are float32; the convolution runs on the normed activations in the
+    compute dtype, which is also what its state keeps, so a cut changes no number.
+
+    Tensor roles: ``conv1``, ``conv2``, ``gate1_weight``, ``gate1_bias``, ``gate2_weight``,
+    ``gate2_bias``."""
+
+    def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: PartSpec = None,
+                 feed_forward: PartSpec = None, conv_taps: int = 0, residual_gate: bool = True,
+                 tensors: Dict[str, str] = None):
+        super().__init__(tensors)
+        if (feed_forward is None) != (norm2 is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.hidden_size, self.conv_taps, self.residual_gate = int(hidden_size), int(conv_taps), bool(residual_gate)
+        self.norm1 = build_part("norm", norm1)
+        self.mixer = build_part("mixer", mixer)
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
+        self.w_conv = [None, None]
+        self.w_gate = [None, None]
+        self.b_gate = [None, None]
+
+    def parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
+
+    def mixer_part(self):
+        return self.mixer
+
+    def _sublayers(self):
+        return (1, 2) if self.feed_forward is not None else (1,)
+
+    def tensor_specs(self):
+        specs = {}
+        for p in self.parts():
+            specs.update(p.tensor_specs())
+        t, w = self.tensor_names, self.hidden_size
+        for i in self._sublayers():
+            if self.conv_taps:
+                specs[t[f"conv{i}"]] = TensorSpec((w, self.conv_taps), MATRIX)
+            if self.residual_gate:
+                specs[t[f"gate{i}_weight"]] = TensorSpec((w, w), MATRIX)
+                specs[t[f"gate{i}_bias"]] = TensorSpec((w,), VECTOR, INIT_ZEROS)
+        return specs
+
+    def state_spec(self):
+        """The mixer's state and, for each convolution, its last ``taps - 1`` inputs (compute dtype)."""
+        spec = dict(self.mixer.state_spec())
+        if self.conv_taps > 1:
+            for i in self._sublayers():
+                spec[f"conv{i}"] = ((self.conv_taps - 1, self.hidden_size), None)
+        return spec
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        for p in self.parts():
+            p.bind(tensors, ops, dtype)
+        t = self.tensor_names
+        ops.check_product_sizes(self.hidden_size, dtype, "residual gate (hidden size)")
+        for i in self._sublayers():
+            if self.conv_taps:      # (taps side by side for each channel, float32: four numbers a channel)
+                self.w_conv[i - 1] = tensors[t[f"conv{i}"]].float().contiguous()
+            if self.residual_gate:
+                self.w_gate[i - 1] = ops.prepare_weight(tensors[t[f"gate{i}_weight"]].contiguous())
+                self.b_gate[i - 1] = tensors[t[f"gate{i}_bias"]].float().contiguous()
+
+    def kernel_libraries(self):
+        return [("stream_ops", None)] + super().kernel_libraries()
+
+    def _fold(self, residual, ctx):
+        pending = getattr(ctx, "pending", None)
+        if pending is not None:
+            self.ops.add_pending(residual, pending)
+            ctx.pending = None
+
+    def _half(self, i, norm, part, residual, ctx, entry, *view):
+        ops, rows = self.ops, residual.shape[0]
+        self._fold(residual, ctx)
+        h = ctx.scratch("block.normed", (rows, self.hidden_size), self.dtype)
+        norm.forward(residual, h)
+        hin = h
+        if self.conv_taps:
+            hin = ctx.scratch("block.convolved", (rows, self.hidden_size), self.dtype)
+            state = entry.state.get(f"conv{i}")
+            ops.causal_conv(h, self.w_conv[i - 1], state, ctx.positions, ctx.row_req, ctx.all_q_start,
+                            ctx.all_req_rows, hin)
+        y = ctx.scratch("block.sublayer_out", (rows, self.hidden_size), torch.float32)
+        if part.writes_output:
+            part.forward_into(hin, y, ctx, *view)
+        else:
+            ops.activation(y, y, "zero")
+            part.forward(hin, y, ctx, *view)
+            self._fold(y, ctx)
+        gate = None
+        if self.residual_gate:
+            gate = ctx.scratch("block.gate", (rows, self.hidden_size), torch.float32)
+            ops.linear_logits(h, self.w_gate[i - 1], gate)
+        ops.gated_add(residual, y, gate, self.b_gate[i - 1])
+
+    def forward(self, residual, ctx, entry):
+        self._half(1, self.norm1, self.mixer, residual, ctx, entry, entry)
+        if self.feed_forward is not None:
+            self._half(2, self.norm2, self.feed_forward, residual, ctx, entry)
+
+    def weight_bytes(self):
+        own = sum(w.numel() * w.element_size() for w in self.w_conv + self.w_gate + self.b_gate if w is not None)
+        return own + sum(p.weight_bytes() for p in self.parts())
+
+
 class TokenEmbedding(Part):
     """``x[r] = table[id_r]`` into the float32 residual stream
     (rust/engine/src/runner/model/qwen2/kernels.rs:46-57)."""
@@ -176,14 +295,71 @@ class TokenEmbedding(Part):
         return 0     # a step reads one row per token, not the table
 
 
+class PairHashEmbedding(Part):
+    """``x[r] = norm(table[id_r] * scale + pairs[row_r])`` into the float32 stream: beside the token's
+    own vector a row of a second table that the token and the one before it in its sequence pick
+    together, ``row = (previous * mul_prev + id * mul_cur) mod buckets``; a sequence's first token
+    takes the row behind the buckets (row number ``buckets``).  The token before a step's first
+    one is per-request state (one integer), so a sequence may be cut anywhere.  ``norm``: a norm
+    part applied to the sum in place (None: none); sum and norm in float32.
+
+    Tensor roles: ``weight [vocab, hidden]``, ``pairs [buckets + 1, hidden]``."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, tensors: Dict[str, str], scale: float = 1.0,
+                 buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0, norm: PartSpec = None):
+        super().__init__(tensors)
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.scale, self.buckets, self.mul_prev, self.mul_cur = float(scale), int(buckets), int(mul_prev), int(mul_cur)
+        self.norm = build_part("norm", norm) if norm is not None else None
+        self.table = self.pairs = None
+        self.state = {}
+
+    def tensor_specs(self):
+        specs = {self.tensor_names["weight"]: TensorSpec((self.vocab_size, self.hidden_size), MATRIX)}
+        if self.buckets:
+            specs[self.tensor_names["pairs"]] = TensorSpec((self.buckets + 1, self.hidden_size), MATRIX)
+        if self.norm is not None:
+            specs.update(self.norm.tensor_specs())
+        return specs
+
+    def state_spec(self):
+        return {"previous_token": ((1,), torch.int32)} if self.buckets else {}
+
+    def attach_state(self, state):
+        self.state = dict(state)
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        self.table = tensors[self.tensor_names["weight"]].contiguous()
+        self.pairs = tensors[self.tensor_names["pairs"]].contiguous() if self.buckets else None
+        if self.norm is not None:
+            self.norm.bind(tensors, ops, dtype)
+            if self.norm.rms_params() is None:
+                raise ValueError(f"{type(self.norm).__name__} is no RMS norm: the embedding's kernel takes one")
+
+    def forward(self, ids, out, ctx):
+        weight, eps = self.norm.rms_params() if self.norm is not None else (None, 0.0)
+        self.ops.embed_pairs(self.table, self.pairs, ids, ctx.positions, ctx.row_req, ctx.all_q_start,
+                             ctx.all_req_rows, self.state.get("previous_token"), self.scale, self.buckets,
+                             self.mul_prev, self.mul_cur, weight, eps, out)
+
+    def kernel_libraries(self):
+        return [("stream_ops", None)]
+
+    def weight_bytes(self):
+        return 0     # a step reads two rows per token, not the tables
+
+
 class LinearHead(Part):
     """``logits = h W^T`` in float32; ``W`` is the embedding table when the
     names coincide (tied), as in rust/engine/src/runner/model/qwen2/engine.rs:299-303
-    and 1312-1319."""
+    and 1312-1319.  ``softcap``: the logits are then bent into ``(-cap, cap)``,
+    ``cap * tanh(logits / cap)``."""
 
-    def __init__(self, vocab_size: int, hidden_size: int, tensors: Dict[str, str]):
+    def __init__(self, vocab_size: int, hidden_size: int, tensors: Dict[str, str], softcap: float = None):
         super().__init__(tensors)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.softcap = None if softcap is None else float(softcap)     # logits <- cap * tanh(logits / cap)
         self.weight = None
 
     def tensor_specs(self):
@@ -209,12 +385,19 @@ class LinearHead(Part):
             if isinstance(h, NormedInput):
                 h = h.tensor()
             self.ops.linear_logits(h, self.weight, out)
+        if self.softcap is not None:
+            self.ops.softcap(out, self.softcap)
+
+    def kernel_libraries(self):
+        return [("stream_ops", None)] if self.softcap is not None else []
 
     def weight_bytes(self):
         return self.weight.numel() * self.weight.element_size()
 
 
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "gated_conv", GatedConvBlock)
+register_part("embedding", "pair_hash_embedding", PairHashEmbedding)
 register_part("block", "sublayer_norm", SublayerNormBlock)
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "linear_head", LinearHead)

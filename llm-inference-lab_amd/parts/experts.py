@@ -8,7 +8,7 @@ import torch
 from ..config.spec import PartSpec
 from ..weights.loader import TensorSpec, MATRIX, VECTOR, INIT_ZEROS
 from .base import FeedForward, NormedInput
-from .feed_forward import interleave_gate_up, pad_columns
+from .feed_forward import interleave_gate_up, pad_columns, pad_rows
 from .registry import register_part, build_part
 
 
@@ -27,6 +27,11 @@ class RoutedExperts(FeedForward):
     tensors: their result is ``h`` itself.  ``shared``: a feed-forward part that every token goes
     through, added to the sum.
 
+    ``scoring="sigmoid"``: the scores are ``sigmoid(z)``, each output by itself, instead of the
+    softmax.  ``expert_form="relu2"``: the experts are ``W_down relu(W_up h)^2`` without a gate
+    matrix.  ``shared_gate=True``: the shared part's result is multiplied by ``sigmoid(w_sg . h)``,
+    one number per token (``shared_gate [1, hidden]``), before it is added.
+
     Tensor roles: ``router [outputs, hidden]``, ``correction [outputs]`` (absent: none), and the
     experts' ``expert_gate``, ``expert_up``, ``expert_down``, each a name with ``{}`` in the place of
     the expert's number.
@@ -38,8 +43,17 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, tensors: Dict[str, str],
                  identity: int = 0, scale: float = 1.0, groups: int = 1, groups_keep: int = 1,
-                 correction: bool = True, shared: Optional[PartSpec] = None):
+                 correction: bool = True, shared: Optional[PartSpec] = None, scoring: str = "softmax",
+                 expert_form: str = "swiglu", shared_gate: bool = False):
         super().__init__(tensors)
+        if scoring not in ("softmax", "sigmoid"):
+            raise ValueError(f"a router scores by 'softmax' or 'sigmoid', got {scoring!r}")
+        if expert_form not in ("swiglu", "relu2"):
+            raise ValueError(f"experts are 'swiglu' or 'relu2' feed-forwards, got {expert_form!r}")
+        if shared_gate and shared is None:
+            raise ValueError("a gate on the shared part needs a shared part")
+        self.scoring, self.expert_form, self.has_shared_gate = scoring, expert_form, bool(shared_gate)
+        self.w_shared_gate = None
         self.hidden_size, self.expert_size = int(hidden_size), int(expert_size)
         self.kernel_size = (self.expert_size + 7) // 8 * 8       # (as in ``SwiGLU``: zeros behind an odd width)
         self.num_experts, self.identity, self.top = int(num_experts), int(identity), int(top)
@@ -59,7 +73,8 @@ class RoutedExperts(FeedForward):
 
     def _expert_names(self, e: int):
         t = self.tensor_names
-        return t["expert_gate"].format(e), t["expert_up"].format(e), t["expert_down"].format(e)
+        gate = t["expert_gate"].format(e) if self.expert_form == "swiglu" else None
+        return gate, t["expert_up"].format(e), t["expert_down"].format(e)
 
     def tensor_specs(self):
         t, w, f = self.tensor_names, self.hidden_size, self.expert_size
@@ -68,10 +83,13 @@ class RoutedExperts(FeedForward):
             specs[t["correction"]] = TensorSpec((self.outputs,), VECTOR, INIT_ZEROS)
         for e in range(self.num_experts):
             gate, up, down = self._expert_names(e)
-            specs[gate], specs[up], specs[down] = (TensorSpec((f, w), MATRIX), TensorSpec((f, w), MATRIX),
-                                                   TensorSpec((w, f), MATRIX))
+            if gate is not None:
+                specs[gate] = TensorSpec((f, w), MATRIX)
+            specs[up], specs[down] = TensorSpec((f, w), MATRIX), TensorSpec((w, f), MATRIX)
         if self.shared is not None:
             specs.update(self.shared.tensor_specs())
+        if self.has_shared_gate:
+            specs[t["shared_gate"]] = TensorSpec((1, w), MATRIX)
         return specs
 
     def bind(self, tensors, ops, dtype):
@@ -84,7 +102,14 @@ class RoutedExperts(FeedForward):
         # Every expert's gate and up rows interleaved as the paired epilogue reads them, the experts
         # one below the other: one matrix, of which an expert is a run of whole strips of rows.
         names = [self._expert_names(e) for e in range(self.num_experts)]
-        if names:
+        if names and self.expert_form == "relu2":
+            # (an expert's up rows in whole strips of 16, its down columns zeros behind an odd width)
+            self.gate_up_rows = (self.expert_size + 15) // 16 * 16
+            self.w_gate_up = ops.prepare_stacked(torch.cat([pad_rows(tensors[u], self.gate_up_rows) for _, u, _ in names],
+                                                           dim=0).contiguous(), self.num_experts)
+            self.w_down = ops.prepare_stacked(torch.cat([pad_columns(tensors[d], self.gate_up_rows) for _, _, d in names],
+                                                        dim=0).contiguous(), self.num_experts)
+        elif names:
             gate_up = [interleave_gate_up(tensors[g], tensors[u]) for g, u, _ in names]
             self.gate_up_rows = gate_up[0].shape[0]
             self.w_gate_up = ops.prepare_stacked(torch.cat(gate_up, dim=0).contiguous(), self.num_experts)
@@ -93,6 +118,8 @@ class RoutedExperts(FeedForward):
                                               self.num_experts)
         if self.shared is not None:
             self.shared.bind(tensors, ops, dtype)
+        if self.has_shared_gate:
+            self.w_shared_gate = ops.prepare_weight(tensors[t["shared_gate"]].contiguous())
 
     takes_normed_input = True
 
@@ -107,33 +134,55 @@ class RoutedExperts(FeedForward):
         weights = ctx.scratch("experts.weights", (rows, top), torch.float32)
         grouped = self.num_experts and getattr(ops, "moe_grouped", None) is not None and ops.moe_grouped(self.dtype)
         plan = None
+        how = {} if self.scoring == "softmax" else dict(scoring=self.scoring)
         if grouped and ops.moe_select_plan_takes(rows, self.outputs):       # few rows: choice and sorting in one launch
             plan = ops.moe_select_plan(logits, self.correction, self.groups, self.groups_keep, self.scale, chosen,
-                                       weights, self.num_experts, ctx.scratch)
+                                       weights, self.num_experts, ctx.scratch, **how)
         else:
-            ops.moe_select(logits, self.correction, self.groups, self.groups_keep, self.scale, chosen, weights)
+            ops.moe_select(logits, self.correction, self.groups, self.groups_keep, self.scale, chosen, weights, **how)
         if grouped:
             self._grouped(h, residual, ctx, chosen, weights, plan)
         elif self.num_experts:
-            act = ctx.scratch("experts.act", (rows, self.kernel_size), self.dtype)
+            relu2 = self.expert_form == "relu2"
+            act = ctx.scratch("experts.act", (rows, self.gate_up_rows if relu2 else self.kernel_size), self.dtype)
             y = ctx.scratch("experts.out", (rows, self.hidden_size), torch.float32)
             for e in range(self.num_experts):
-                ops.linear_swiglu(h, ops.stacked_member(self.w_gate_up, e), act)
+                if relu2:
+                    ops.linear_relu2(h, ops.stacked_member(self.w_gate_up, e), act)
+                else:
+                    ops.linear_swiglu(h, ops.stacked_member(self.w_gate_up, e), act)
                 ops.linear_logits(act, ops.stacked_member(self.w_down, e), y)
                 ops.moe_add_chosen(residual, y, chosen, weights, e, e + 1)
             if self.identity:
                 ops.moe_add_chosen(residual, h, chosen, weights, self.num_experts, self.outputs)
         elif self.identity:
             ops.moe_add_chosen(residual, h, chosen, weights, self.num_experts, self.outputs)
-        if self.shared is not None:
+        if self.shared is not None and not self.has_shared_gate:
             self.shared.forward(h, residual, ctx)
+        elif self.shared is not None:
+            y = ctx.scratch("experts.shared_out", (rows, self.hidden_size), torch.float32)
+            if self.shared.writes_output:
+                self.shared.forward_into(h, y, ctx)
+            else:
+                ops.activation(y, y, "zero")
+                self.shared.forward(h, y, ctx)
+                if getattr(ctx, "pending", None) is not None:       # (pieces the shared part left belong to y)
+                    ops.add_pending(y, ctx.pending)
+                    ctx.pending = None
+            g = ctx.scratch("experts.shared_gate", (rows, 1), torch.float32)
+            ops.linear_logits(h, self.w_shared_gate, g)
+            ops.gated_add(residual, y, g, None)
 
     def _grouped(self, h, residual, ctx, chosen, weights, plan=None):
         ops = self.ops
         if plan is None:
             plan = ops.moe_plan(chosen, self.num_experts, ctx.scratch)
-        act = ctx.scratch("experts.act", (plan.capacity, self.kernel_size), self.dtype)
-        ops.moe_gate_up(h, self.w_gate_up, plan, act)
+        if self.expert_form == "relu2":
+            act = ctx.scratch("experts.act", (plan.capacity, self.gate_up_rows), self.dtype)
+            ops.moe_up_relu2(h, self.w_gate_up, plan, act)
+        else:
+            act = ctx.scratch("experts.act", (plan.capacity, self.kernel_size), self.dtype)
+            ops.moe_gate_up(h, self.w_gate_up, plan, act)
         y = ctx.scratch("experts.out", (plan.capacity, self.hidden_size), torch.float32)
         ops.moe_down(act, self.w_down, plan, y)
         ops.moe_combine(residual, y, plan, chosen, weights, self.num_experts, h)     # (identity outputs too)
@@ -153,7 +202,7 @@ class RoutedExperts(FeedForward):
         """What a step of many rows reads: every expert.  (A step of few rows reads the experts
         its rows chose.)"""
         total = 0
-        for w in (self.w_router, self.w_gate_up, self.w_down):
+        for w in (self.w_router, self.w_gate_up, self.w_down, self.w_shared_gate):
             if w is not None:
                 total += w.numel() * w.element_size()
         return total + (self.shared.weight_bytes() if self.shared is not None else 0)

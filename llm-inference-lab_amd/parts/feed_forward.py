@@ -40,6 +40,15 @@ def pad_columns(w: torch.Tensor, columns: int) -> torch.Tensor:
     return out
 
 
+def pad_rows(w: torch.Tensor, rows: int) -> torch.Tensor:
+    """``w [n, k]`` with zero rows below it up to ``rows``."""
+    if w.shape[0] == rows:
+        return w.contiguous()
+    out = torch.zeros((rows, w.shape[1]), dtype=w.dtype, device=w.device)
+    out[:w.shape[0]] = w
+    return out
+
+
 class SwiGLU(FeedForward):
     """``residual += (silu(h Wg^T) * (h Wu^T)) Wd^T`` with ``silu(z) = z / (1 +
     exp(-z))``; accumulators, the sigmoid and the product in float32.
@@ -117,6 +126,7 @@ class DenseFeedForward(FeedForward):
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"a dense feed-forward takes the activations {self.ACTIVATIONS}, got '{activation}'")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.kernel_size = (self.intermediate_size + 7) // 8 * 8      # (as in ``SwiGLU``: zeros behind an odd width)
         self.activation = activation
         self.w_up = self.w_down = None
 
@@ -127,19 +137,18 @@ class DenseFeedForward(FeedForward):
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         ops.check_product_sizes(self.hidden_size, dtype, "feed-forward (hidden size)")
-        ops.check_product_sizes(self.intermediate_size, dtype, "feed-forward (intermediate size)")
         t = self.tensor_names
-        self.w_up = ops.prepare_weight(tensors[t["up_weight"]].contiguous())
-        self.w_down = ops.prepare_weight(tensors[t["down_weight"]].contiguous())
+        self.w_up = ops.prepare_weight(pad_rows(tensors[t["up_weight"]], self.kernel_size))
+        self.w_down = ops.prepare_weight(pad_columns(tensors[t["down_weight"]], self.kernel_size))
 
     def _activated(self, h, ctx):
         rows = h.shape[0]
-        act = ctx.scratch("dense_ffn.act", (rows, self.intermediate_size), self.dtype)
+        act = ctx.scratch("dense_ffn.act", (rows, self.kernel_size), self.dtype)
         fused = getattr(self.ops, "linear_relu2", None) if self.activation == "relu2" else None
         if fused is not None:
             fused(h, self.w_up, act)            # the activation is the first product's epilogue
             return act
-        sums = ctx.scratch("dense_ffn.sums", (rows, self.intermediate_size), torch.float32)
+        sums = ctx.scratch("dense_ffn.sums", (rows, self.kernel_size), torch.float32)
         self.ops.linear_logits(h, self.w_up, sums)
         self.ops.activation(sums, act, self.activation)
         return act

@@ -18,25 +18,31 @@ class RMSNorm(Norm):
     reference rounds once more, before the weight product; in float32 the two
     are the same).  ``size`` and ``eps`` come from the caller.  ``weight_offset``: the stored
     tensor is the scale less this constant (a weight kept around zero has ``weight_offset=1``:
-    ``w = 1 + stored``); the sum is taken once, in float32, when the part is bound."""
+    ``w = 1 + stored``); the sum is taken once, in float32, when the part is bound.  ``scalar``: the
+    stored weight is ONE number for all coordinates (a tensor without axes); it is spread over the
+    width when the part is bound, so every kernel that takes an RMS norm's weight serves it."""
 
     folds_pending = True
     keeps_launches = True
 
-    def __init__(self, size: int, eps: float, tensors: Dict[str, str], weight_offset: float = 0.0):
+    def __init__(self, size: int, eps: float, tensors: Dict[str, str], weight_offset: float = 0.0,
+                 scalar: bool = False):
         super().__init__(tensors)
         self.size = int(size)
         self.eps = float(eps)
         self.weight_offset = float(weight_offset)
+        self.scalar = bool(scalar)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self):
-        return {self.tensor_names["weight"]: TensorSpec((self.size,), VECTOR,
+        return {self.tensor_names["weight"]: TensorSpec(() if self.scalar else (self.size,), VECTOR,
                                                         INIT_NORMAL if self.weight_offset else INIT_NORM)}
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         self.weight = tensors[self.tensor_names["weight"]].contiguous()
+        if self.scalar:
+            self.weight = self.weight.reshape(1).expand(self.size).contiguous()
         if self.weight_offset:
             self.weight = (self.weight.float() + self.weight_offset).contiguous()
 

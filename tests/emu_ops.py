@@ -60,7 +60,8 @@ class EmuOps:
                 "fused_norm_swiglu", "fused_norm_logits", "rope_inplace", "rope_kv_write",
                 "paged_attention", "argmax", "sample", "layernorm", "layernorm_add", "activation",
                 "project_norm_write", "sink_window_attention", "gla_decay", "gla_scan", "gla_output",
-                "gate_heads", "add_row_vector", "moe_select", "moe_add_chosen")
+                "gate_heads", "add_row_vector", "moe_select", "moe_add_chosen", "embed_pairs", "causal_conv",
+                "gated_add", "latent_norm_write", "head_products", "softcap")
 
     def __init__(self, device="cpu", fuse=True):
         self.device = torch.device(device)
@@ -385,15 +386,16 @@ class EmuOps:
     def moe_grouped(self, dtype):
         return False
 
-    def moe_select(self, logits, correction, groups, groups_keep, scale, chosen, weights):
-        """Per row: softmax of the logits, the choice value (score + correction), the kept groups by
-        their best choice value, the ``top`` best of their members; ties to the smaller index."""
+    def moe_select(self, logits, correction, groups, groups_keep, scale, chosen, weights, scoring="softmax"):
+        """Per row: softmax (or, ``scoring="sigmoid"``, the sigmoid) of the logits, the choice value
+        (score + correction), the kept groups by their best choice value, the ``top`` best of their
+        members; ties to the smaller index."""
         self._count("moe_select")
         rows, outputs = logits.shape
         top = chosen.shape[1]
         z = logits.float()
         e = torch.exp(z - z.max(-1, keepdim=True).values)
-        s = e / e.sum(-1, keepdim=True)
+        s = e / e.sum(-1, keepdim=True) if scoring == "softmax" else torch.sigmoid(z)
         c = s + correction.float()
         per = outputs // groups
         best = c.view(rows, groups, per).max(-1).values
@@ -410,6 +412,112 @@ class EmuOps:
             chosen[:, k] = e_k.to(torch.int32)
             weights[:, k] = s[torch.arange(rows), e_k] * scale
             c[torch.arange(rows), e_k] = -float("inf")
+
+    # ------------------------------- hashed pairs, short convolution, gates, latent attention
+    def embed_pairs(self, table, pairs, ids, positions, row_req, q_start, req_rows, previous, scale, buckets,
+                    mul_prev, mul_cur, norm_weight, eps, out):
+        """``out[r] = norm(table[id_r] * scale + pairs[row_r])``; the token before a request's first
+        row of the step comes from ``previous[slot]``, which then takes the request's last token."""
+        self._count("embed_pairs")
+        rows = out.shape[0]
+        x = table[ids[:rows].long()].float() * scale
+        if buckets:
+            last = {}
+            for r in range(rows):
+                b = int(row_req[r])
+                slot = int(req_rows[b])
+                if int(positions[r]) == 0:
+                    at = buckets
+                else:
+                    before = int(ids[r - 1]) if r > int(q_start[b]) else int(previous[slot, 0])
+                    at = (before * mul_prev + int(ids[r]) * mul_cur) % buckets
+                x[r] += pairs[at].float()
+                last[slot] = int(ids[r])
+            for slot, token in last.items():
+                previous[slot, 0] = token
+        if norm_weight is not None:
+            x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        out.copy_(x)
+
+    def causal_conv(self, h, weight, state, positions, row_req, q_start, req_rows, out):
+        """``out_t = h_t + sum_j weight[:, j] h_(t - taps + 1 + j)`` over the positions of each request;
+        inputs from before the step come from ``state [slots, taps - 1, width]`` (the latest last),
+        which then takes the request's latest inputs."""
+        self._count("causal_conv")
+        rows, taps = h.shape[0], weight.shape[1]
+        w = weight.float()
+        hf = h.float()
+        res = hf.clone()
+        starts = {}
+        for r in range(rows):
+            b = int(row_req[r])
+            first = int(q_start[b])
+            starts.setdefault(b, first)
+            slot = int(req_rows[b])
+            for j in range(taps):
+                back = taps - 1 - j                 # how many positions behind row r
+                if back == 0:
+                    src = hf[r]
+                elif r - back >= first:
+                    src = hf[r - back]
+                elif state is not None:              # (zeros stand there before the sequence's start)
+                    src = state[slot, taps - 1 - (back - (r - first))].float()
+                else:
+                    continue
+                res[r] += w[:, j] * src
+        out.copy_(res.to(out.dtype))
+        if state is None or taps <= 1:
+            return
+        for b, first in starts.items():
+            n = sum(1 for r in range(rows) if int(row_req[r]) == b)
+            slot = int(req_rows[b])
+            joined = torch.cat([state[slot].float(), hf[first:first + n]], dim=0)
+            state[slot] = joined[-(taps - 1):].to(state.dtype)
+
+    def gated_add(self, x, y, gate, bias):
+        """``x += y * sigmoid(gate + bias)``: ``gate [rows, width]`` or one number a row ``[rows, 1]``
+        (None: ``x += y``), all float32."""
+        self._count("gated_add")
+        if gate is None:
+            x += y
+            return
+        g = gate.float() + (bias.float() if bias is not None else 0.0)
+        x += y * torch.sigmoid(g)
+
+    def latent_norm_write(self, proj, q_rank, q_laid, kv_rank, latent, gates, q_norm, c_norm, eps, cq_out, gate_out,
+                          k_cache, v_cache, page_size, positions, row_req, block_table):
+        """From ``proj [rows, q_laid + latent + gates]`` float32: the query's latent (RMS norm over its
+        first ``q_rank`` numbers, weight ``q_norm``) into ``cq_out``; the cached latent (RMS norm over
+        ``kv_rank`` numbers, weight ``c_norm``) into the row's place of both page tensors; the heads'
+        gates as they are into ``gate_out``."""
+        self._count("latent_norm_write")
+        rows = cq_out.shape[0]
+        p = proj.float()
+
+        def normed(v, n, w):
+            return v / torch.sqrt((v[:, :n] ** 2).sum(-1, keepdim=True) / n + eps) * w.float()
+        cq_out.copy_(normed(p[:, :q_laid], q_rank, q_norm).to(cq_out.dtype))
+        c = normed(p[:, q_laid:q_laid + latent], kv_rank, c_norm).to(k_cache.dtype)
+        if gates:
+            gate_out.copy_(p[:, q_laid + latent:q_laid + latent + gates])
+        for r in range(rows):
+            pos = int(positions[r])
+            page = int(block_table[int(row_req[r]), pos // page_size])
+            o = pos % page_size
+            k_cache[page, 0, o] = c[r]
+            cache_layout.value_quads(v_cache[page])[0, o >> 2, :, o & 3] = c[r]
+
+    def head_products(self, x, w, out):
+        """``out[r, a, :] = w[a] x[r, a, :]`` for a stack ``w [heads, n, k]``; sums in float32."""
+        self._count("head_products")
+        heads, n, k = w.shape
+        rows = x.shape[0]
+        res = torch.einsum("rak,ank->ran", x.float().view(rows, heads, k), w.float())
+        out.copy_(res.reshape(rows, heads * n).to(out.dtype))
+
+    def softcap(self, x, cap):
+        self._count("softcap")
+        x.copy_(cap * torch.tanh(x / cap))
 
     def moe_add_chosen(self, resid, src, chosen, weights, first, last):
         """``resid[r] += sum over k with first <= chosen[r, k] < last of weights[r, k] * src[r]``."""

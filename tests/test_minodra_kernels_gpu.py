@@ -1,0 +1,183 @@
+"""The kernels that Minodra brought, each alone against its plain PyTorch reference (tests/emu_ops.py):
+the embedding with hashed token pairs, the short causal convolution with its per-request state, the
+gated sum, the soft cap, the latent's norm and cache write, the per-head products, the sigmoid router."""
+import pytest
+import torch
+
+from emu_ops import EmuOps
+from llm_inference_lab_amd.cache import layout as cache_layout
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llm_inference_lab_amd.kernels.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+@pytest.fixture(scope="module")
+def emu():
+    return EmuOps("cpu")
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def ints(values):
+    return torch.tensor(values, dtype=torch.int32)
+
+
+def step_description(portions, starts, slots):
+    """positions, row_req, q_start, req_rows of a step whose request b brings ``portions[b]`` rows from
+    position ``starts[b]`` on and lives in slot ``slots[b]``."""
+    positions, row_req, q_start = [], [], [0]
+    for b, (n, s) in enumerate(zip(portions, starts)):
+        positions += list(range(s, s + n))
+        row_req += [b] * n
+        q_start.append(q_start[-1] + n)
+    return ints(positions), ints(row_req), ints(q_start), ints(slots)
+
+
+def on(device, *tensors):
+    return [None if t is None else t.to(device) for t in tensors]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden,vocab,buckets,norm", [(64, 50, 13, True), (100, 300, 1021, True), (24, 9, 1, False),
+                                                       (72, 40, 0, True)])
+def test_embed_pairs_over_steps(ops, emu, dtype, hidden, vocab, buckets, norm):
+    """Three steps of three requests in slots 2, 0, 3: portions, single tokens, a request that starts
+    in the second step; the slots carry the last token from step to step."""
+    table, pairs = rnd((vocab, hidden), dtype, 1), rnd((buckets + 1, hidden), dtype, 2) if buckets else None
+    weight = (1 + 0.3 * rnd((1,), torch.float32, 3)).expand(hidden).contiguous() if norm else None
+    state_e, state_g = torch.zeros(4, 1, dtype=torch.int32), torch.zeros(4, 1, dtype=torch.int32, device=DEV)
+    g = torch.Generator().manual_seed(5)
+    steps = [([5, 1], [0, 0], [2, 0]), ([1, 3, 2], [5, 1, 0], [2, 0, 3]), ([1, 1, 6], [6, 4, 2], [2, 0, 3])]
+    for portions, starts, slots in steps:
+        rows = sum(portions)
+        ids = torch.randint(0, vocab, (rows,), generator=g).int()
+        desc = step_description(portions, starts, slots)
+        want = torch.empty(rows, hidden)
+        emu.embed_pairs(table, pairs, ids, *desc, state_e if buckets else None, 3.5, buckets, 127, 7, weight, 1e-5, want)
+        got = torch.empty(rows, hidden, device=DEV)
+        ops.embed_pairs(*on(DEV, table, pairs, ids, *desc), state_g if buckets else None, 3.5, buckets, 127, 7,
+                        None if weight is None else weight.to(DEV), 1e-5, got)
+        assert (got.cpu() - want).abs().max() <= 2e-5 * max(1.0, float(want.abs().max()))
+        assert torch.equal(state_g.cpu(), state_e)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,taps", [(64, 4), (100, 2), (24, 7), (40, 1)])
+def test_causal_conv_over_steps(ops, emu, dtype, width, taps):
+    """Portions shorter and longer than the taps, single tokens, a sequence's start inside a step: the
+    outputs and the slots after every step."""
+    weight = rnd((width, taps), torch.float32, 1, 0.7)
+    keep = max(taps - 1, 0)
+    state_e = torch.zeros(4, keep, width, dtype=dtype) if keep else None
+    state_g = torch.zeros(4, keep, width, dtype=dtype, device=DEV) if keep else None
+    steps = [([2, 1], [0, 0], [1, 3]), ([1, 9, 3], [2, 1, 0], [1, 3, 0]), ([1, 1, 1], [3, 10, 3], [1, 3, 0]),
+             ([taps + 3, 2], [4, 11], [1, 3])]
+    for n, (portions, starts, slots) in enumerate(steps):
+        rows = sum(portions)
+        h = rnd((rows, width), dtype, 10 + n)
+        desc = step_description(portions, starts, slots)
+        want = torch.empty(rows, width, dtype=dtype)
+        emu.causal_conv(h, weight, state_e, *desc, want)
+        got = torch.empty(rows, width, dtype=dtype, device=DEV)
+        ops.causal_conv(h.to(DEV), weight.to(DEV), state_g, *on(DEV, *desc), got)
+        tol = 1e-5 if dtype == torch.float32 else 1.0 / 64
+        assert (got.cpu().float() - want.float()).abs().max() <= tol * max(1.0, float(want.float().abs().max()))
+        if keep:
+            assert torch.equal(state_g.cpu(), state_e)
+
+
+@pytest.mark.parametrize("rows,width,cols,bias", [(1, 64, 64, True), (7, 100, 100, True), (5, 66, 1, False),
+                                                  (33, 320, 320, False), (3, 8, None, False)])
+def test_gated_add(ops, emu, rows, width, cols, bias):
+    x, y = rnd((rows, width), torch.float32, 1), rnd((rows, width), torch.float32, 2)
+    gate = rnd((rows, cols), torch.float32, 3, 2.0) if cols else None
+    b = rnd((width,), torch.float32, 4) if bias else None
+    want = x.clone()
+    emu.gated_add(want, y, gate, b)
+    got = x.to(DEV)
+    ops.gated_add(got, *on(DEV, y, gate, b))
+    assert (got.cpu() - want).abs().max() <= 1e-5
+
+
+def test_softcap(ops, emu):
+    x = rnd((5, 333), torch.float32, 1, 40.0)
+    want = x.clone()
+    emu.softcap(want, 30.0)
+    got = x.to(DEV)
+    ops.softcap(got, 30.0)
+    assert (got.cpu() - want).abs().max() <= 1e-4
+    assert float(got.abs().max()) <= 30.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("q_rank,kv_rank,gates", [(24, 32, 3), (20, 40, 0), (128, 96, 6), (7, 5, 1)])
+def test_latent_norm_write(ops, emu, dtype, q_rank, kv_rank, gates):
+    q_laid, latent, page = (q_rank + 7) // 8 * 8, (kv_rank + 31) // 32 * 32, 16
+    portions, starts, slots = [5, 1, 20], [14, 33, 0], [0, 1, 2]
+    positions, row_req, _, _ = step_description(portions, starts, slots)
+    rows = sum(portions)
+    proj = rnd((rows, q_laid + latent + gates), torch.float32, 1, 2.0)
+    proj[:, q_rank:q_laid] = 0
+    proj[:, q_laid + kv_rank:q_laid + latent] = 0
+    q_w, c_w = torch.zeros(q_laid), torch.zeros(latent)
+    q_w[:q_rank], c_w[:kv_rank] = 1 + 0.3 * rnd((q_rank,), torch.float32, 2), 1 + 0.3 * rnd((kv_rank,), torch.float32, 3)
+    table = torch.tensor([[3, 7, 0], [1, 5, 2], [6, 4, 8]], dtype=torch.int32)
+    caches = [torch.zeros(9, 1, page, latent, dtype=dtype) for _ in range(2)]
+    cq, gate = torch.empty(rows, q_laid, dtype=dtype), torch.empty(rows, max(gates, 1))[:, :gates].contiguous()
+    emu.latent_norm_write(proj, q_rank, q_laid, kv_rank, latent, gates, q_w, c_w, 1e-5, cq, gate, *caches, page,
+                          positions, row_req, table)
+    g_caches = [torch.zeros(9, 1, page, latent, dtype=dtype, device=DEV) for _ in range(2)]
+    g_cq, g_gate = torch.empty(rows, q_laid, dtype=dtype, device=DEV), torch.empty(rows, gates, device=DEV)
+    ops.latent_norm_write(proj.to(DEV), q_rank, q_laid, kv_rank, latent, gates, q_w.to(DEV), c_w.to(DEV), 1e-5, g_cq,
+                          g_gate if gates else None, *g_caches, page, *on(DEV, positions, row_req, table))
+    tol = 1e-5 if dtype == torch.float32 else 1.0 / 64
+    assert (g_cq.cpu().float() - cq.float()).abs().max() <= tol * 4
+    for got, want in zip(g_caches, caches):
+        assert (got.cpu().float() - want.float()).abs().max() <= tol * 4
+    # both page tensors hold the same vectors, one row by row and one in quads of keys
+    quads = cache_layout.value_quads(g_caches[1].cpu())
+    assert torch.equal(quads.permute(0, 1, 2, 4, 3).reshape(9, 1, page, latent), g_caches[0].cpu())
+    if gates:
+        assert torch.equal(g_gate.cpu(), gate)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,heads,n,k", [(1, 6, 96, 32), (37, 3, 32, 96), (16, 2, 80, 64), (5, 4, 24, 40),
+                                            (70, 5, 272, 128), (3, 1, 7, 9)])
+def test_head_products(ops, emu, dtype, rows, heads, n, k):
+    x, w = rnd((rows, heads * k), dtype, 1), rnd((heads, n, k), dtype, 2, k ** -0.5)
+    want = torch.empty(rows, heads * n, dtype=dtype)
+    emu.head_products(x, w, want)
+    for plain in (False, True):
+        ops.force_plain_windowed_attention(plain)
+        try:
+            got = torch.zeros(rows, heads * n, dtype=dtype, device=DEV)
+            ops.head_products(x.to(DEV), w.to(DEV), got)
+        finally:
+            ops.force_plain_windowed_attention(False)
+        tol = 2e-5 if dtype == torch.float32 else 1.0 / 64
+        assert (got.cpu().float() - want.float()).abs().max() <= tol * max(1.0, float(want.float().abs().max()))
+
+
+@pytest.mark.parametrize("rows,outputs,top", [(1, 8, 4), (9, 5, 1), (40, 64, 6), (3, 100, 8), (17, 7, 7)])
+def test_sigmoid_router_choice(ops, emu, rows, outputs, top):
+    logits = rnd((rows, outputs), torch.float32, 1, 2.0)
+    correction = rnd((outputs,), torch.float32, 2, 0.3)
+    want_c, want_w = torch.zeros(rows, top, dtype=torch.int32), torch.zeros(rows, top)
+    emu.moe_select(logits, correction, 1, 1, 1.0, want_c, want_w, scoring="sigmoid")
+    got_c, got_w = torch.zeros(rows, top, dtype=torch.int32, device=DEV), torch.zeros(rows, top, device=DEV)
+    ops.moe_select(logits.to(DEV), correction.to(DEV), 1, 1, 1.0, got_c, got_w, scoring="sigmoid")
+    assert torch.equal(got_c.cpu(), want_c)
+    assert (got_w.cpu() - want_w).abs().max() <= 1e-6
+    # the weights are the scores themselves: not normalised, the correction left out
+    assert torch.allclose(got_w.cpu(), torch.sigmoid(logits).gather(1, want_c.long()), atol=1e-6)
