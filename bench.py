@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S]
                     [--shape 0.5b|7b|32b] [--layers L] [--dtype bf16|f32]
     python bench.py --mixed [--shape 7b] [--requests 64] [--chunk 512] [--outputs 64]
-    python bench.py --design vivevik|ruvalorn [--size small|medium|large] [--context 2048]
+    python bench.py --design vivevik|ruvalorn|minodra [--size small|medium|large] [--context 2048]
 
 Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
 batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
@@ -44,6 +44,9 @@ layer's keys and values) at layer sizes of real models, beside the Qwen2 decoder
 width, heads, feed-forward width and number of layers; one JSON line, a record per size.
 ``--design ruvalorn``: the same for the Ruvalorn design (windowed attention whose values are its
 keys, a gate per head, mixtures of experts behind a grouped router, some layers run twice).
+``--design minodra``: the same for the Minodra design (attention over one cached latent vector per
+token, a short convolution in front of every sublayer, gated sums into the stream, mixtures of
+squared-ReLU experts behind a sigmoid router in every other layer).
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -195,6 +198,47 @@ def ruvalorn_flops(cfg, tokens):
     return total + 2 * w * cfg.vocab
 
 
+# ``--design minodra``: per size (query latent, cached latent, experts, expert width, chosen per token,
+# shared expert's width).  The experts have no gate matrix, so chosen * expert width + shared width is
+# one and a half times the dense feed-forward's width: a token does the Qwen2 decoder's arithmetic in
+# the feed-forwards.  Even layers have the dense feed-forward, odd layers the mixture; four taps.
+MINODRA_SIZES = {"small": (384, 128, 32, 768, 8, 1152), "medium": (768, 256, 32, 1536, 8, 4224),
+                 "large": (1536, 256, 32, 2560, 8, 7936)}
+
+
+def minodra_config(size):
+    import llm_inference_lab_amd as lab
+    width, heads, _, dim, ff, layers = DESIGN_SIZES[size]
+    q_rank, kv_rank, experts, expert_ff, top, shared = MINODRA_SIZES[size]
+    listed = []
+    for i in range(layers):
+        mixer = dict(heads=heads, dim=dim, vdim=dim, q_rank=q_rank, kv_rank=kv_rank, scale=dim ** -0.5)
+        mlp = dict(kind="dense", ff=ff) if i % 2 == 0 else dict(
+            kind="moe", expert=dict(ff=expert_ff), shared=dict(ff=shared), router=dict(experts=experts, top=top))
+        listed.append(dict(type="latent_attention", mixer=mixer, mlp=mlp))
+    return lab.MinodraConfig.from_dict(dict(
+        architecture="Minodra", vocab=DESIGN_VOCAB, width=width, norm=dict(eps=1e-6), layers=listed, canon=dict(taps=4),
+        embedding=dict(scale=12.0, bigram=dict(buckets=65521, mul_prev=127, mul_cur=7)), logit_softcap=30.0))
+
+
+def minodra_flops(cfg, tokens):
+    """Multiply-adds times two of one prompt of ``tokens`` positions as the engine computes them: the
+    queries are taken into the cached vector's coordinates, so a (query, key) pair of a head costs the
+    latent's width twice."""
+    w, total = cfg.width, 0
+    pairs = tokens * (tokens + 1) // 2
+    for l in cfg.layers:
+        total += tokens * 2 * (w * (l.q_rank + l.kv_rank + l.heads) + l.q_rank * l.heads * l.dim
+                               + l.heads * l.kv_rank * (l.dim + l.vdim) + l.heads * l.vdim * w + w * w)
+        total += 4 * pairs * l.heads * l.kv_rank
+        f = l.mlp
+        if f is not None and f.kind == "dense":
+            total += tokens * (6 * w * f.ff + 2 * w * w)
+        elif f is not None:
+            total += tokens * (2 * w * f.experts + 4 * w * f.ff * f.top + 4 * w * (f.shared_ff or 0) + 2 * w * w)
+    return total + 2 * w * cfg.vocab
+
+
 def design_run(args, bracket=None):
     """``--design vivevik``: both models at each size, one after the other on the same GPU.
     ``--only-model``, ``--only-prefill`` / ``--only-decode`` and ``--batch`` narrow the run (for
@@ -214,7 +258,7 @@ def design_run(args, bracket=None):
                                               num_key_value_heads=kv, head_dim=dim, tie_word_embeddings=True))
         record[size] = {"width": width, "heads": heads, "kv_heads": kv, "head_dim": dim, "ff": ff, "layers": layers,
                         "context": context, "window": DESIGN_WINDOW}
-        design = ruvalorn_config(size) if args.design == "ruvalorn" else vivevik_config(size)
+        design = {"ruvalorn": ruvalorn_config, "minodra": minodra_config, "vivevik": vivevik_config}[args.design](size)
         for label, cfg in ((args.design, design), ("qwen2", qwen)):
             if args.only_model and label != args.only_model:
                 continue
@@ -231,6 +275,7 @@ def design_run(args, bracket=None):
             runs = Runs(engine, view, context, args.dtype, args.samples, bracket)
             flops = (vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else
                      ruvalorn_flops(cfg, args.prefill_tokens) if label == "ruvalorn" else
+                     minodra_flops(cfg, args.prefill_tokens) if label == "minodra" else
                      prefill_flops(cfg, args.prefill_tokens))
             out = {"weight_bytes_per_step": engine.weight_bytes_per_step()}
             if not args.only_decode:
@@ -762,10 +807,10 @@ def main():
                     help="fix a choice of the kernels for the whole run, to compare variants: a keyword of "
                          "engine.ops.debug.force, values separated by ':' (attention_splits=64:8, "
                          "attention_merge_kernel=64, gemm_tile=129)")
-    ap.add_argument("--design", choices=["vivevik", "ruvalorn"], default=None,
+    ap.add_argument("--design", choices=["vivevik", "ruvalorn", "minodra"], default=None,
                     help="throughput of another design beside the Qwen2 decoder of equal size")
     ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default=None, help="--design: one size only")
-    ap.add_argument("--only-model", choices=["vivevik", "ruvalorn", "qwen2"], default=None, help="--design: one of the two models only")
+    ap.add_argument("--only-model", choices=["vivevik", "ruvalorn", "minodra", "qwen2"], default=None, help="--design: one of the two models only")
     ap.add_argument("--only-decode", action="store_true", help="--design: decode at --batch only, no prefill")
     ap.add_argument("--side", choices=["7b", "32b", "f32", "peaks"], help=argparse.SUPPRESS)
     args = ap.parse_args()

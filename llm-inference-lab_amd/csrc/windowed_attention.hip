@@ -529,7 +529,10 @@ __global__ __launch_bounds__(64) void sink_window_attention_merge_kernel(MfmaArg
 
 // Whether the matrix-core kernel takes these sizes at all.
 extern "C" int llmlab_sink_window_attention_has_mfma(int dtype, int D, int E, int page_size) {
-  return !g_force_plain && dtype == DT_BF16 && D % 32 == 0 && D <= 128 && E % 16 == 0 && E <= 128 && page_size % 16 == 0;
+  if (g_force_plain || dtype != DT_BF16 || D % 32 != 0 || E % 16 != 0 || page_size % 16 != 0) return 0;
+  // (keys and values up to 128 wide in any combination; wider ones, up to 256, where both are of
+  // one width: the latent form, whose values are its keys)
+  return (D <= 128 && E <= 128) || (D == E && D <= 256);
 }
 
 template <int DC>
@@ -546,6 +549,16 @@ static void launch_mfma(int EBv, int which, dim3 grid, dim3 block, hipStream_t s
 }
 
 static void launch_mfma_any(int D, int E, int which, dim3 grid, dim3 block, hipStream_t stream, const MfmaArgs& a) {
+#define LLMLAB_MFMA_SQUARE(DCV)                                                                                          \
+  case DCV:                                                                                                             \
+    if (which == 0) hipLaunchKernelGGL((sink_window_attention_mfma_kernel<DCV, 2 * DCV>), grid, block, 0, stream, a);     \
+    else hipLaunchKernelGGL((sink_window_attention_grouped_kernel<DCV, 2 * DCV>), grid, block, 0, stream, a);            \
+    return;
+  if (D > 128) {
+    switch (D / 32) { LLMLAB_MFMA_SQUARE(5) LLMLAB_MFMA_SQUARE(6) LLMLAB_MFMA_SQUARE(7) LLMLAB_MFMA_SQUARE(8) }
+    return;
+  }
+#undef LLMLAB_MFMA_SQUARE
   switch (D / 32) {
     case 1: launch_mfma<1>(E / 16, which, grid, block, stream, a); break;
     case 2: launch_mfma<2>(E / 16, which, grid, block, stream, a); break;

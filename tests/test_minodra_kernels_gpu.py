@@ -181,3 +181,37 @@ def test_sigmoid_router_choice(ops, emu, rows, outputs, top):
     assert (got_w.cpu() - want_w).abs().max() <= 1e-6
     # the weights are the scores themselves: not normalised, the correction left out
     assert torch.allclose(got_w.cpu(), torch.sigmoid(logits).gather(1, want_c.long()), atol=1e-6)
+
+
+@pytest.mark.parametrize("latent", [32, 96, 160, 256])
+@pytest.mark.parametrize("heads", [3, 16, 20])
+def test_attention_over_one_cached_vector_per_token(ops, emu, latent, heads):
+    """The attention kernels in the latent form (one key/value head, values = keys, a sink): a portion
+    of a prompt behind a history, a whole prompt and two decoding requests in one step, by the
+    matrix-core kernels and by the plain one, against the reference key by key."""
+    dtype, page = torch.bfloat16, 16
+    portions, starts, slots = [40, 1, 23, 1], [37, 150, 0, 16], [0, 1, 2, 3]
+    positions, row_req, q_start, _ = step_description(portions, starts, slots)
+    rows = sum(portions)
+    table = torch.randperm(48, generator=torch.Generator().manual_seed(3)).int().view(4, 12)
+    vectors = rnd((48, page, latent), dtype, 1)
+    k_cache = vectors.view(48, 1, page, latent).clone()
+    v_cache = torch.zeros_like(k_cache)
+    cache_layout.value_quads(v_cache)[:, 0] = vectors.view(48, page // 4, 4, latent).permute(0, 1, 3, 2)
+    q = rnd((rows, heads * latent), dtype, 2, 3.0 / latent ** 0.5)
+    sink = rnd((heads,), torch.float32, 4, 2.0)
+    want = torch.zeros(rows, heads * latent, dtype=dtype)
+    emu.sink_window_attention(q, heads, 1, latent, latent, k_cache, v_cache, table, page, positions, row_req, None, 0,
+                              sink, 0.7, want)
+    for plain in (False, True):
+        ops.force_plain_windowed_attention(plain)
+        try:
+            long_from = ops.windowed_attention_long_rows(dtype, latent, latent, page)
+            assert bool(long_from) == (not plain)
+            got = torch.zeros(rows, heads * latent, dtype=dtype, device=DEV)
+            ops.sink_window_attention(q.to(DEV), heads, 1, latent, latent, k_cache.to(DEV), v_cache.to(DEV), table.to(DEV),
+                                      page, positions.to(DEV), row_req.to(DEV), None, 0, sink.to(DEV), 0.7, got,
+                                      q_start.to(DEV), long_from, 3, 200)
+        finally:
+            ops.force_plain_windowed_attention(False)
+        assert (got.cpu().float() - want.float()).abs().max() <= 2e-2, (latent, heads, plain)
