@@ -1,6 +1,7 @@
 // Operations on the float32 residual stream around the sublayers of a layer, for gfx950:
 //   embed_pairs     x[r] = norm(table[id] * scale + pairs[hash(previous id, id)])
 //   causal_conv     out_t = h_t + sum_j w[:, j] h_(t - taps + 1 + j) over the positions of a request
+//   norm_conv       the RMS norm of the stream's rows and that convolution over them in one launch
 //   gated_add       x += y * sigmoid(gate + bias)
 //   softcap         x = cap * tanh(x / cap)
 // What a request's earlier steps left (its last token, the last inputs of a convolution) lives in
@@ -154,6 +155,127 @@ extern "C" int llmlab_causal_conv(const void* h, int dtype, const float* w, int 
                          (float*)state, row_req, q_start, req_rows, width);
   }
   LLMLAB_LAUNCH_CHECK("causal_conv");
+  return 0;
+}
+
+// ------------------------------------------------------------------ norm and convolution in one
+// h = x / sqrt(mean(x^2) + eps) * g (rounded to T), conv = h + sum_j w[:, j] h_(t - taps + 1 + j):
+// the RMS norm of the float32 stream's rows and the convolution over them in one launch.  One
+// block a row.  A row's block norms the row itself and, again, the up to TAPS - 1 rows of its
+// request before it in the step (the same sums in the same order as those rows' own blocks, so
+// the same numbers); what lies before the step comes from the slots.  Every load of the second
+// pass is unconditional (a row or a slot place that is not wanted is read at a place that is
+// and dropped), so that they travel together.  own_state: every request brings one row, and the
+// row's block moves its slot on after it has read it (a thread owns its channels); otherwise
+// causal_conv_state_kernel does that from h in a launch of its own.
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void norm_conv_kernel(const float* __restrict__ x, const void* __restrict__ g,
+                                                        int g_bf16, float eps, const float* __restrict__ w,
+                                                        T* __restrict__ state, const int* __restrict__ row_req,
+                                                        const int* __restrict__ q_start,
+                                                        const int* __restrict__ req_rows, T* __restrict__ h,
+                                                        T* __restrict__ conv, int width, int own_state) {
+  constexpr int KEEP = TAPS - 1;
+  __shared__ float red[4][TAPS];
+  __shared__ float s_inv[TAPS];
+  const int r = blockIdx.x;
+  const int b = row_req[r];
+  const int first = q_start[b];
+  const int inside = min(r - first, KEEP);            // rows of this request before r that the taps reach
+  T* st = state && KEEP > 0 ? state + (size_t)req_rows[b] * KEEP * width : nullptr;
+  float ss[TAPS];
+#pragma unroll
+  for (int k = 0; k < TAPS; ++k) ss[k] = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float v[TAPS];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) v[k] = x[(size_t)(r - min(k, inside)) * width + c];
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) ss[k] = fmaf(v[k], v[k], ss[k]);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < TAPS; ++k) ss[k] = wave_sum(ss[k]);
+  if (lane == 0) {
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) red[wave][k] = ss[k];
+  }
+  __syncthreads();
+  if (threadIdx.x < TAPS) {
+    const float t = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+    s_inv[threadIdx.x] = 1.0f / sqrtf(t / (float)width + eps);
+  }
+  __syncthreads();
+  float inv[TAPS];
+#pragma unroll
+  for (int k = 0; k < TAPS; ++k) inv[k] = s_inv[k];
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float xv[TAPS], sv[TAPS], wv[TAPS];
+    const float gc = load_vec(g, g_bf16, c);
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) xv[k] = x[(size_t)(r - min(k, inside)) * width + c];
+#pragma unroll
+    for (int k = 1; k < TAPS; ++k)                    // place in the slot of the input `k` positions back
+      sv[k] = st ? to_float(st[(size_t)min(max(KEEP - (k - inside), 0), KEEP - 1) * width + c]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wv[j] = w[(size_t)c * TAPS + j];
+    const T own = from_float<T>(xv[0] * inv[0] * gc);
+    float acc = to_float(own);
+    acc = fmaf(wv[TAPS - 1], to_float(own), acc);
+    T hk[TAPS];
+    hk[0] = own;
+#pragma unroll
+    for (int k = 1; k < TAPS; ++k) {
+      hk[k] = k <= inside ? from_float<T>(xv[k] * inv[k] * gc) : from_float<T>(sv[k]);
+      acc = fmaf(wv[TAPS - 1 - k], to_float(hk[k]), acc);
+    }
+    h[(size_t)r * width + c] = own;
+    conv[(size_t)r * width + c] = from_float<T>(acc);
+    if (own_state && st) {
+#pragma unroll
+      for (int s = 0; s < KEEP; ++s) st[(size_t)s * width + c] = hk[KEEP - 1 - s];
+    }
+  }
+}
+
+template <typename T>
+static void launch_norm_conv(int taps, int rows, hipStream_t stream, const float* x, const void* g, int g_bf16, float eps,
+                             const float* w, T* state, const int* row_req, const int* q_start, const int* req_rows, T* h,
+                             T* conv, int width, int own_state) {
+#define LLMLAB_NORM_CONV(N)                                                                                             \
+  case N:                                                                                                               \
+    hipLaunchKernelGGL((norm_conv_kernel<T, N>), dim3(rows), dim3(256), 0, stream, x, g, g_bf16, eps, w, state, row_req, \
+                       q_start, req_rows, h, conv, width, own_state);                                                   \
+    break;
+  switch (taps) {
+    LLMLAB_NORM_CONV(1) LLMLAB_NORM_CONV(2) LLMLAB_NORM_CONV(3) LLMLAB_NORM_CONV(4)
+    LLMLAB_NORM_CONV(5) LLMLAB_NORM_CONV(6) LLMLAB_NORM_CONV(7) LLMLAB_NORM_CONV(8)
+  }
+#undef LLMLAB_NORM_CONV
+}
+
+// one_row_each: every request of the step brings exactly one row (the host knows).
+extern "C" int llmlab_norm_conv(const float* x, const void* g, int g_dtype, float eps, const float* w, int taps,
+                                void* state, const int* row_req, const int* q_start, const int* req_rows, void* h,
+                                void* conv, int dtype, int rows, int width, int one_row_each, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && width > 0 && taps >= 1 && taps <= 8, "norm_conv: 1 to 8 taps, got rows=%d width=%d taps=%d",
+                 rows, width, taps);
+  LLMLAB_REQUIRE(row_req && q_start && (taps == 1 || (state && req_rows)), "norm_conv: the step's description is missing");
+  if (rows == 0) return 0;
+  if (dtype == DT_BF16) {
+    launch_norm_conv<bf16_t>(taps, rows, stream, x, g, g_dtype == DT_BF16, eps, w, (bf16_t*)state, row_req, q_start,
+                             req_rows, (bf16_t*)h, (bf16_t*)conv, width, one_row_each);
+    if (taps > 1 && !one_row_each)
+      hipLaunchKernelGGL(causal_conv_state_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)h, taps,
+                         (bf16_t*)state, row_req, q_start, req_rows, width);
+  } else {
+    launch_norm_conv<float>(taps, rows, stream, x, g, g_dtype == DT_BF16, eps, w, (float*)state, row_req, q_start,
+                            req_rows, (float*)h, (float*)conv, width, one_row_each);
+    if (taps > 1 && !one_row_each)
+      hipLaunchKernelGGL(causal_conv_state_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)h, taps,
+                         (float*)state, row_req, q_start, req_rows, width);
+  }
+  LLMLAB_LAUNCH_CHECK("norm_conv");
   return 0;
 }
 

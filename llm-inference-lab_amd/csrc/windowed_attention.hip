@@ -504,25 +504,54 @@ __global__ __launch_bounds__(64) void sink_window_attention_grouped_kernel(MfmaA
 }
 
 // out[r, h] = sum_z exp(m_z - M) o_z / sum_z exp(m_z - M) l_z over the shares of the row's keys.
+// One wave per (row, head).  The shares' maxima and sums are read once, a lane a share; the
+// shares' weights exp(m_z - M) lie in LDS, and the loop over the shares' partial outputs has no
+// branch (an empty share weighs zero and its numbers are dropped), so its loads travel together.
+constexpr int MERGE_MAX_SPLITS = 256;
 __global__ __launch_bounds__(64) void sink_window_attention_merge_kernel(MfmaArgs a, int E) {
+  __shared__ float s_w[MERGE_MAX_SPLITS];
   const int r = blockIdx.x, h = blockIdx.y;
   const int b = a.row_req[r];
   if (a.long_from > 0 && a.q_start[b + 1] - a.q_start[b] >= a.long_from) return;
   const size_t first = ((size_t)r * a.n_heads + h) * a.splits;
+  constexpr int PER_LANE = MERGE_MAX_SPLITS / 64;
+  float m[PER_LANE], l[PER_LANE];
   float big = NEG_INF;
-  for (int z = 0; z < a.splits; ++z) big = fmaxf(big, a.part_ml[(first + z) * 2]);
-  float den = 0.f;
-  for (int z = 0; z < a.splits; ++z) {
-    const float m = a.part_ml[(first + z) * 2];
-    if (m != NEG_INF) den += __expf(m - big) * a.part_ml[(first + z) * 2 + 1];
+#pragma unroll
+  for (int i = 0; i < PER_LANE; ++i) {
+    const int z = threadIdx.x + 64 * i;
+    const int at = min(z, a.splits - 1);
+    const float mz = a.part_ml[(first + at) * 2], lz = a.part_ml[(first + at) * 2 + 1];
+    m[i] = z < a.splits ? mz : NEG_INF;
+    l[i] = lz;
+    big = fmaxf(big, m[i]);
   }
+  big = wave_max(big);
+  float den = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER_LANE; ++i) {
+    const float w = m[i] != NEG_INF ? __expf(m[i] - big) : 0.f;
+    if (w != 0.f) den = fmaf(w, l[i], den);
+    s_w[threadIdx.x + 64 * i] = w;
+  }
+  den = wave_sum(den);
+  __syncthreads();
+  const float inv = 1.0f / den;
   for (int e = threadIdx.x; e < E; e += 64) {
     float acc = 0.f;
-    for (int z = 0; z < a.splits; ++z) {
-      const float m = a.part_ml[(first + z) * 2];
-      if (m != NEG_INF) acc = fmaf(__expf(m - big), a.part_o[(first + z) * E + e], acc);
+    int z = 0;
+    for (; z + 4 <= a.splits; z += 4) {
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = a.part_o[(first + z + j) * E + e];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc = fmaf(s_w[z + j], s_w[z + j] != 0.f ? o[j] : 0.f, acc);
     }
-    a.out[((size_t)r * a.n_heads + h) * E + e] = (bf16_t)(acc / den);
+    for (; z < a.splits; ++z) {
+      const float o = a.part_o[(first + z) * E + e];
+      acc = fmaf(s_w[z], s_w[z] != 0.f ? o : 0.f, acc);
+    }
+    a.out[((size_t)r * a.n_heads + h) * E + e] = (bf16_t)(acc * inv);
   }
 }
 
@@ -613,7 +642,7 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
       if (workspace == nullptr) splits = 1;
       else if (splits * per_split > workspace_floats) splits = (long)(workspace_floats / per_split);
       if (splits < 1) splits = 1;
-      if (splits > 65535) splits = 65535;
+      if (splits > MERGE_MAX_SPLITS) splits = MERGE_MAX_SPLITS;
       a.splits = (int)splits;
       a.part_o = workspace;
       a.part_ml = workspace ? workspace + (size_t)rows * n_heads * splits * E : nullptr;
@@ -715,9 +744,11 @@ extern "C" int llmlab_latent_norm_write(const float* proj, int ld, int rows, int
 // Plain kernel (any sizes, both dtypes): a block per (row, head), the head's K numbers in LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void head_products_kernel(const T* __restrict__ x, const T* __restrict__ w,
-                                                            T* __restrict__ out, int heads, int N, int K) {
+                                                            T* __restrict__ out, int heads, int N, int K,
+                                                            const float* __restrict__ gate) {
   extern __shared__ float xs[];
   const int r = blockIdx.x, a = blockIdx.y;
+  const float scale = gate ? 1.f / (1.f + __expf(-gate[(size_t)r * heads + a])) : 1.f;
   const T* xr = x + ((size_t)r * heads + a) * K;
   for (int k = threadIdx.x; k < K; k += blockDim.x) xs[k] = to_float(xr[k]);
   __syncthreads();
@@ -727,7 +758,7 @@ __global__ __launch_bounds__(256) void head_products_kernel(const T* __restrict_
     float s = 0.f;
     for (int k = lane; k < K; k += 64) s = fmaf(to_float(wr[k]), xs[k], s);
     s = wave_sum(s);
-    if (lane == 0) out[((size_t)r * heads + a) * N + n] = from_float<T>(s);
+    if (lane == 0) out[((size_t)r * heads + a) * N + n] = from_float<T>(s * scale);
   }
 }
 
@@ -738,7 +769,7 @@ constexpr int HP_TILES = 4;
 
 __global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                  bf16_t* __restrict__ out, int rows, int heads, int N,
-                                                                 int K) {
+                                                                 int K, const float* __restrict__ gate) {
   const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4, wave = threadIdx.x >> 6;
   const int r0 = blockIdx.x * 16, a = blockIdx.y;
   const int n_first = (blockIdx.z * 4 + wave) * HP_TILES * 16;
@@ -747,6 +778,7 @@ __global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* _
   const bool row_ok = r < rows;
   const bf16_t* xr = x + ((size_t)(row_ok ? r : rows - 1) * heads + a) * K + 8 * g4;
   const bf16_t* wa = w + (size_t)a * N * K;
+  const float gv = gate ? gate[(size_t)(row_ok ? r : rows - 1) * heads + a] : 0.f;
   floatx4 acc[HP_TILES];
   const bf16_t* wr[HP_TILES];
 #pragma unroll
@@ -764,19 +796,22 @@ __global__ __launch_bounds__(256) void head_products_mfma_kernel(const bf16_t* _
     }
   }
   if (!row_ok) return;
+  const float scale = gate ? 1.f / (1.f + __expf(-gv)) : 1.f;
 #pragma unroll
   for (int t = 0; t < HP_TILES; ++t) {
     const int n = n_first + 16 * t + 4 * g4;
     if (n >= N) continue;
     bf16x4 o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = (bf16_t)acc[t][i];
+    for (int i = 0; i < 4; ++i) o[i] = (bf16_t)(acc[t][i] * scale);
     *(bf16x4*)(out + ((size_t)r * heads + a) * N + n) = o;
   }
 }
 
+// gate: float32 [rows, heads] or null; head a of row r is multiplied by sigmoid(gate[r, a]) before
+// the one rounding.
 extern "C" int llmlab_head_products(const void* x, const void* w, void* out, int dtype, int rows, int heads, int N,
-                                    int K, hipStream_t stream) {
+                                    int K, const float* gate, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0 && K <= 12288,
                  "head_products: bad sizes rows=%d heads=%d N=%d K=%d", rows, heads, N, K);
   if (rows == 0) return 0;
@@ -784,13 +819,13 @@ extern "C" int llmlab_head_products(const void* x, const void* w, void* out, int
       ((uintptr_t)out & 7) == 0) {
     dim3 grid((rows + 15) / 16, heads, (N + 4 * HP_TILES * 16 - 1) / (4 * HP_TILES * 16));
     hipLaunchKernelGGL(head_products_mfma_kernel, grid, dim3(256), 0, stream, (const bf16_t*)x, (const bf16_t*)w,
-                       (bf16_t*)out, rows, heads, N, K);
+                       (bf16_t*)out, rows, heads, N, K, gate);
   } else if (dtype == DT_BF16) {
     hipLaunchKernelGGL(head_products_kernel<bf16_t>, dim3(rows, heads), dim3(256), K * sizeof(float), stream,
-                       (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)out, heads, N, K);
+                       (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)out, heads, N, K, gate);
   } else {
     hipLaunchKernelGGL(head_products_kernel<float>, dim3(rows, heads), dim3(256), K * sizeof(float), stream,
-                       (const float*)x, (const float*)w, (float*)out, heads, N, K);
+                       (const float*)x, (const float*)w, (float*)out, heads, N, K, gate);
   }
   LLMLAB_LAUNCH_CHECK("head_products");
   return 0;

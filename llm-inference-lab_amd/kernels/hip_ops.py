@@ -1066,7 +1066,7 @@ class HipOps:
                     _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_latent_norm_write.restype = _c_int
                 lib.llmlab_head_products.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                                     _c_ptr]
+                                                     _c_ptr, _c_ptr]
                 lib.llmlab_head_products.restype = _c_int
             elif kind == "stream_ops":
                 lib.llmlab_embed_pairs.argtypes = [
@@ -1076,6 +1076,9 @@ class HipOps:
                 lib.llmlab_causal_conv.argtypes = [_c_ptr, _c_int, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                                    _c_ptr, _c_int, _c_int, _c_ptr]
                 lib.llmlab_causal_conv.restype = _c_int
+                lib.llmlab_norm_conv.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                                                 _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
+                lib.llmlab_norm_conv.restype = _c_int
                 lib.llmlab_gated_add.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]
                 lib.llmlab_gated_add.restype = _c_int
                 lib.llmlab_softcap.argtypes = [_c_ptr, _c_float, _c_size, _c_ptr]
@@ -1554,6 +1557,42 @@ class HipOps:
                    self._ptr(row_req), self._ptr(q_start), self._ptr(req_rows), self._ptr(out), rows, width,
                    self._stream(), lib=lib)
 
+    NORM_CONV_MAX_TAPS = 8
+
+    def norm_conv(self, x, norm_weight, eps: float, weight, state, row_req, q_start, req_rows, h, out,
+                  one_row_each: bool) -> None:
+        """``h = rmsnorm(x) * norm_weight`` and ``out_t = h_t + sum_j weight[:, j] h_(t - taps + 1 + j)`` in
+        one launch: the norm of the float32 stream's rows and ``causal_conv`` over them (up to
+        ``NORM_CONV_MAX_TAPS`` taps).  ``one_row_each``: every request of the step brings exactly one
+        row; then the slots are moved on in the same launch."""
+        lib = self._mixer_lib("stream_ops")
+        self._need(x, "residual stream", torch.float32)
+        self._need(norm_weight, "norm weight")
+        self._need(h, "normed rows")
+        self._need(out, "convolution output", h.dtype)
+        self._need(weight, "convolution taps", torch.float32)
+        rows, width = x.shape
+        taps = weight.shape[1]
+        if tuple(weight.shape) != (width, taps) or tuple(out.shape) != (rows, width) or tuple(h.shape) != (rows, width) \
+                or norm_weight.numel() != width:
+            raise ValueError(f"norm_conv: stream {tuple(x.shape)}, norm weight {tuple(norm_weight.shape)}, taps "
+                             f"{tuple(weight.shape)}, outputs {tuple(h.shape)} and {tuple(out.shape)}")
+        if not 1 <= taps <= self.NORM_CONV_MAX_TAPS:
+            raise ValueError(f"norm_conv: 1 to {self.NORM_CONV_MAX_TAPS} taps, got {taps}")
+        if taps > 1:
+            self._need(state, "convolution state", h.dtype)
+            if tuple(state.shape[1:]) != (taps - 1, width):
+                raise ValueError(f"norm_conv: state {tuple(state.shape)} does not hold {taps - 1} inputs of {width}")
+        for t, name, least in ((row_req, "row -> request map", rows), (q_start, "request row starts", 2),
+                               (req_rows, "request slots", 1)):
+            self._need(t, name, torch.int32)
+            if t.numel() < least:
+                raise ValueError(f"norm_conv: {name} is too short")
+        self._call(lib.llmlab_norm_conv, self._ptr(x), self._ptr(norm_weight), _dt(norm_weight), float(eps),
+                   self._ptr(weight), taps, self._ptr(state) if taps > 1 else None, self._ptr(row_req), self._ptr(q_start),
+                   self._ptr(req_rows), self._ptr(h), self._ptr(out), _dt(h), rows, width, 1 if one_row_each else 0,
+                   self._stream(), lib=lib)
+
     def gated_add(self, x, y, gate, bias) -> None:
         """``x += y * sigmoid(gate + bias)``, all float32: ``gate [rows, width]``, or ``[rows, 1]`` for
         one number a row; ``bias [width]`` or None; ``gate`` None: ``x += y``."""
@@ -1615,9 +1654,10 @@ class HipOps:
                    _dt(cq_out), page_size, self._ptr(positions), self._ptr(row_req), self._ptr(block_table),
                    block_table.stride(0), self._stream(), lib=lib)
 
-    def head_products(self, x, w, out) -> None:
+    def head_products(self, x, w, out, gate=None) -> None:
         """``out[r, a, :] = w[a] x[r, a, :]`` for a stack of matrices ``w [heads, n, k]``: ``x [rows, heads *
-        k]``, ``out [rows, heads * n]``, all of one kernel dtype; sums in float32."""
+        k]``, ``out [rows, heads * n]``, all of one kernel dtype; sums in float32.  ``gate [rows, heads]``
+        float32: head ``a`` of row ``r`` times ``sigmoid(gate[r, a])``, in float32 before the rounding."""
         lib = self._mixer_lib("windowed_attention")
         self._need(x, "head inputs")
         self._need(w, "head matrices", x.dtype)
@@ -1626,8 +1666,12 @@ class HipOps:
         rows = x.shape[0]
         if tuple(x.shape) != (rows, heads * k) or tuple(out.shape) != (rows, heads * n):
             raise ValueError(f"head_products: x {tuple(x.shape)}, matrices {tuple(w.shape)}, out {tuple(out.shape)}")
+        if gate is not None:
+            self._need(gate, "head gates", torch.float32)
+            if tuple(gate.shape) != (rows, heads):
+                raise ValueError(f"head_products: gates {tuple(gate.shape)} for {rows} rows of {heads} heads")
         self._call(lib.llmlab_head_products, self._ptr(x), self._ptr(w), self._ptr(out), _dt(x), rows, heads, n, k,
-                   self._stream(), lib=lib)
+                   self._ptr(gate), self._stream(), lib=lib)
 
     def argmax(self, logits, out, one_pass: bool = True) -> None:
         """``out[r]`` = the largest logit's index (the smallest among equals; -1 for a row

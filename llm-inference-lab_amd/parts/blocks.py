@@ -167,6 +167,8 @@ class GatedConvBlock(Block):
     Tensor roles: ``conv1``, ``conv2``, ``gate1_weight``, ``gate1_bias``, ``gate2_weight``,
     ``gate2_bias``."""
 
+    fuse_norm_conv = True      # (False: the norm and the convolution as launches of their own)
+
     def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: PartSpec = None,
                  feed_forward: PartSpec = None, conv_taps: int = 0, residual_gate: bool = True,
                  tensors: Dict[str, str] = None):
@@ -234,17 +236,36 @@ class GatedConvBlock(Block):
             self.ops.add_pending(residual, pending)
             ctx.pending = None
 
+    def _norm_conv_fits(self, norm) -> bool:
+        """Norm and convolution in one launch: an RMS norm, and no more taps than that kernel has."""
+        ops = self.ops
+        return (self.fuse_norm_conv and hasattr(norm, "rms_params") and hasattr(ops, "norm_conv")
+                and self.conv_taps <= getattr(ops, "NORM_CONV_MAX_TAPS", 0))
+
     def _half(self, i, norm, part, residual, ctx, entry, *view):
         ops, rows = self.ops, residual.shape[0]
         self._fold(residual, ctx)
         h = ctx.scratch("block.normed", (rows, self.hidden_size), self.dtype)
-        norm.forward(residual, h)
         hin = h
+        fused = self.conv_taps and self._norm_conv_fits(norm)
+        if not fused:
+            norm.forward(residual, h)
         if self.conv_taps:
             hin = ctx.scratch("block.convolved", (rows, self.hidden_size), self.dtype)
             state = entry.state.get(f"conv{i}")
-            ops.causal_conv(h, self.w_conv[i - 1], state, ctx.positions, ctx.row_req, ctx.all_q_start,
-                            ctx.all_req_rows, hin)
+            if fused:
+                # (whether every request brings one row is not a matter of the number of rows)
+                weight, eps = norm.rms_params()
+                launch = lambda: ops.norm_conv(residual, weight, eps, self.w_conv[i - 1], state, ctx.row_req,
+                                               ctx.all_q_start, ctx.all_req_rows, h, hin, ctx.n_rows == ctx.n_reqs)
+                live = getattr(ops, "live", None)
+                if live is not None:
+                    live(launch)
+                else:
+                    launch()
+            else:
+                ops.causal_conv(h, self.w_conv[i - 1], state, ctx.positions, ctx.row_req, ctx.all_q_start,
+                                ctx.all_req_rows, hin)
         y = ctx.scratch("block.sublayer_out", (rows, self.hidden_size), torch.float32)
         if part.writes_output:
             part.forward_into(hin, y, ctx, *view)

@@ -139,9 +139,7 @@ class LatentAttention(Mixer):
         else:
             attend()
         heads = ctx.scratch("latent_attention.heads", (rows, a * self.value_dim), self.dtype)
-        ops.head_products(mixed, self.w_value, heads)
-        if gate is not None:
-            ops.gate_heads(heads, gate, a, self.value_dim, self.output_gate)
+        ops.head_products(mixed, self.w_value, heads, gate)       # (the heads' sigmoid gates ride on the product)
         ops.linear_logits(heads, self.w_o, out)
 
     def forward(self, h, residual, ctx, entry):

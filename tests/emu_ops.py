@@ -60,7 +60,7 @@ class EmuOps:
                 "fused_norm_swiglu", "fused_norm_logits", "rope_inplace", "rope_kv_write",
                 "paged_attention", "argmax", "sample", "layernorm", "layernorm_add", "activation",
                 "project_norm_write", "sink_window_attention", "gla_decay", "gla_scan", "gla_output",
-                "gate_heads", "add_row_vector", "moe_select", "moe_add_chosen", "embed_pairs", "causal_conv",
+                "gate_heads", "add_row_vector", "moe_select", "moe_add_chosen", "embed_pairs", "causal_conv", "norm_conv",
                 "gated_add", "latent_norm_write", "head_products", "softcap")
 
     def __init__(self, device="cpu", fuse=True):
@@ -474,6 +474,18 @@ class EmuOps:
             joined = torch.cat([state[slot].float(), hf[first:first + n]], dim=0)
             state[slot] = joined[-(taps - 1):].to(state.dtype)
 
+    NORM_CONV_MAX_TAPS = 8
+
+    def norm_conv(self, x, norm_weight, eps, weight, state, row_req, q_start, req_rows, h, out, one_row_each):
+        """The RMS norm of the stream's rows into ``h`` and ``causal_conv`` over them into ``out``."""
+        self._count("norm_conv")
+        if one_row_each and x.shape[0] != len({int(b) for b in row_req[:x.shape[0]]}):
+            raise ValueError("norm_conv: one_row_each, but a request brings several rows")
+        xf = x.float()
+        h.copy_((xf / torch.sqrt((xf * xf).mean(-1, keepdim=True) + eps) * norm_weight.float()).to(h.dtype))
+        self.causal_conv(h, weight, state, None, row_req, q_start, req_rows, out)
+        self.calls["causal_conv"] -= 1              # (one launch, counted above)
+
     def gated_add(self, x, y, gate, bias):
         """``x += y * sigmoid(gate + bias)``: ``gate [rows, width]`` or one number a row ``[rows, 1]``
         (None: ``x += y``), all float32."""
@@ -507,12 +519,15 @@ class EmuOps:
             k_cache[page, 0, o] = c[r]
             cache_layout.value_quads(v_cache[page])[0, o >> 2, :, o & 3] = c[r]
 
-    def head_products(self, x, w, out):
-        """``out[r, a, :] = w[a] x[r, a, :]`` for a stack ``w [heads, n, k]``; sums in float32."""
+    def head_products(self, x, w, out, gate=None):
+        """``out[r, a, :] = w[a] x[r, a, :]`` for a stack ``w [heads, n, k]``; sums in float32; with
+        ``gate [rows, heads]``, head ``a`` of row ``r`` times ``sigmoid(gate[r, a])``."""
         self._count("head_products")
         heads, n, k = w.shape
         rows = x.shape[0]
         res = torch.einsum("rak,ank->ran", x.float().view(rows, heads, k), w.float())
+        if gate is not None:
+            res = res * torch.sigmoid(gate.float()).view(rows, heads, 1)
         out.copy_(res.reshape(rows, heads * n).to(out.dtype))
 
     def softcap(self, x, cap):

@@ -1,6 +1,6 @@
 """The kernels that Minodra brought, each alone against its plain PyTorch reference (tests/emu_ops.py):
-the embedding with hashed token pairs, the short causal convolution with its per-request state, the
-gated sum, the soft cap, the latent's norm and cache write, the per-head products, the sigmoid router."""
+the embedding with hashed token pairs, the short causal convolution with its per-request state (alone, and in one launch with the norm
+in front of it), the gated sum, the soft cap, the latent's norm and cache write, the per-head products, the sigmoid router."""
 import pytest
 import torch
 
@@ -96,6 +96,47 @@ def test_causal_conv_over_steps(ops, emu, dtype, width, taps):
             assert torch.equal(state_g.cpu(), state_e)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,taps", [(64, 4), (100, 2), (24, 7), (40, 1), (896, 4), (72, 8)])
+def test_norm_conv_over_steps(ops, emu, dtype, width, taps):
+    """The norm of the stream's rows and the convolution over them in one launch: portions shorter
+    and longer than the taps, single tokens, a sequence's start inside a step, steps in which every
+    request brings one row (the launch that moves the slots on itself) between steps of portions; the
+    normed rows, the outputs and the slots after every step, and the slots bit by bit against the
+    two launches the one replaces."""
+    weight = rnd((width, taps), torch.float32, 1, 0.7)
+    norm_w = (1 + 0.3 * rnd((1,), torch.float32, 3)).expand(width).contiguous().to(dtype)
+    keep = max(taps - 1, 0)
+    state_e = torch.zeros(4, keep, width, dtype=dtype) if keep else None
+    state_g = torch.zeros(4, keep, width, dtype=dtype, device=DEV) if keep else None
+    state_2 = torch.zeros(4, keep, width, dtype=dtype, device=DEV) if keep else None
+    steps = [([2, 1], [0, 0], [1, 3]), ([1, 1], [2, 1], [1, 3]), ([1, 9, 3], [3, 2, 0], [1, 3, 0]),
+             ([1, 1, 1], [4, 11, 3], [1, 3, 0]), ([1, 1, 1], [5, 12, 4], [1, 3, 0]), ([taps + 3, 2], [6, 13], [1, 3]),
+             ([1], [5], [0])]
+    for n, (portions, starts, slots) in enumerate(steps):
+        rows = sum(portions)
+        x = rnd((rows, width), torch.float32, 10 + n, 3.0)
+        _, row_req, q_start, req_rows = step_description(portions, starts, slots)
+        single = all(p == 1 for p in portions)
+        want_h, want = torch.empty(rows, width, dtype=dtype), torch.empty(rows, width, dtype=dtype)
+        emu.norm_conv(x, norm_w, 1e-5, weight, state_e, row_req, q_start, req_rows, want_h, want, single)
+        got_h, got = torch.empty(rows, width, dtype=dtype, device=DEV), torch.empty(rows, width, dtype=dtype, device=DEV)
+        ops.norm_conv(x.to(DEV), norm_w.to(DEV), 1e-5, weight.to(DEV), state_g, *on(DEV, row_req, q_start, req_rows),
+                      got_h, got, single)
+        two_h, two = torch.empty_like(got_h), torch.empty_like(got)
+        ops.rmsnorm(x.to(DEV), norm_w.to(DEV), 1e-5, two_h)
+        ops.causal_conv(two_h, weight.to(DEV), state_2, None, *on(DEV, row_req, q_start, req_rows), two)
+        tol = 1e-5 if dtype == torch.float32 else 1.0 / 64
+        for a, b in ((got_h, want_h), (got, want), (two, want)):
+            assert (a.cpu().float() - b.float()).abs().max() <= tol * max(1.0, float(b.float().abs().max()))
+        if keep:
+            assert (state_g.cpu().float() - state_e.float()).abs().max() <= tol * max(1.0, float(state_e.float().abs().max()))
+            # a slot holds the request's normed rows themselves
+            for b, slot in enumerate(slots):
+                last = int(q_start[b + 1]) - 1
+                assert torch.equal(state_g[slot, keep - 1], got_h[last])
+
+
 @pytest.mark.parametrize("rows,width,cols,bias", [(1, 64, 64, True), (7, 100, 100, True), (5, 66, 1, False),
                                                   (33, 320, 320, False), (3, 8, None, False)])
 def test_gated_add(ops, emu, rows, width, cols, bias):
@@ -156,17 +197,18 @@ def test_latent_norm_write(ops, emu, dtype, q_rank, kv_rank, gates):
                                             (70, 5, 272, 128), (3, 1, 7, 9)])
 def test_head_products(ops, emu, dtype, rows, heads, n, k):
     x, w = rnd((rows, heads * k), dtype, 1), rnd((heads, n, k), dtype, 2, k ** -0.5)
-    want = torch.empty(rows, heads * n, dtype=dtype)
-    emu.head_products(x, w, want)
-    for plain in (False, True):
-        ops.force_plain_windowed_attention(plain)
-        try:
-            got = torch.zeros(rows, heads * n, dtype=dtype, device=DEV)
-            ops.head_products(x.to(DEV), w.to(DEV), got)
-        finally:
-            ops.force_plain_windowed_attention(False)
-        tol = 2e-5 if dtype == torch.float32 else 1.0 / 64
-        assert (got.cpu().float() - want.float()).abs().max() <= tol * max(1.0, float(want.float().abs().max()))
+    for gate in (None, rnd((rows, heads), torch.float32, 3, 2.0)):
+        want = torch.empty(rows, heads * n, dtype=dtype)
+        emu.head_products(x, w, want, gate)
+        for plain in (False, True):
+            ops.force_plain_windowed_attention(plain)
+            try:
+                got = torch.zeros(rows, heads * n, dtype=dtype, device=DEV)
+                ops.head_products(x.to(DEV), w.to(DEV), got, None if gate is None else gate.to(DEV))
+            finally:
+                ops.force_plain_windowed_attention(False)
+            tol = 2e-5 if dtype == torch.float32 else 1.0 / 64
+            assert (got.cpu().float() - want.float()).abs().max() <= tol * max(1.0, float(want.float().abs().max()))
 
 
 @pytest.mark.parametrize("rows,outputs,top", [(1, 8, 4), (9, 5, 1), (40, 64, 6), (3, 100, 8), (17, 7, 7)])
