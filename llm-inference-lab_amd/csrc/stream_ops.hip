@@ -163,37 +163,82 @@ extern "C" int llmlab_causal_conv(const void* h, int dtype, const float* w, int 
 // the RMS norm of the float32 stream's rows and the convolution over them in one launch.  One
 // block a row.  A row's block norms the row itself and, again, the up to TAPS - 1 rows of its
 // request before it in the step (the same sums in the same order as those rows' own blocks, so
-// the same numbers); what lies before the step comes from the slots.  Every load of the second
-// pass is unconditional (a row or a slot place that is not wanted is read at a place that is
-// and dropped), so that they travel together.  own_state: every request brings one row, and the
-// row's block moves its slot on after it has read it (a thread owns its channels); otherwise
-// causal_conv_state_kernel does that from h in a launch of its own.
-template <typename T, int TAPS>
-__global__ __launch_bounds__(256) void norm_conv_kernel(const float* __restrict__ x, const void* __restrict__ g,
-                                                        int g_bf16, float eps, const float* __restrict__ w,
-                                                        T* __restrict__ state, const int* __restrict__ row_req,
-                                                        const int* __restrict__ q_start,
-                                                        const int* __restrict__ req_rows, T* __restrict__ h,
-                                                        T* __restrict__ conv, int width, int own_state) {
+// the same numbers); what lies before the step comes from the slots.  A thread takes NC_PER
+// channels at a time, and every load of a round is unconditional (a row or a slot place that is
+// not wanted is read at a place that is, and dropped), so that they travel together: a row
+// that fits one round (width <= threads x NC_PER) costs one trip to memory, with the slot's
+// inputs, the taps and the norm's weight asked for before the sums are reduced.  own_state:
+// every request brings one row (row r is request r), and the row's block moves its slot on
+// after it has read it (a thread owns its channels); otherwise causal_conv_state_kernel does
+// that from h in a launch of its own.  NC_PER 1 serves few rows no wider than a block: the
+// straight-line code of a block that runs once is fetched as it runs, and a quarter of the code
+// is a quarter of that wait (8 rows of 896: 9.5 us with four channels a thread, 6.8 with one;
+// the simplest kernels take 2.8).
+template <typename T, int TAPS, int NC_PER>
+struct NormConvLoads {
+  float x[NC_PER][TAPS], s[NC_PER][TAPS], w[NC_PER][TAPS], g[NC_PER];
+};
+
+template <typename T, int TAPS, int NC_PER>
+__device__ __forceinline__ void nc_load_x(NormConvLoads<T, TAPS, NC_PER>& v, const float* __restrict__ x, int r, int inside,
+                                          int width, int c0, int stride) {
+#pragma unroll
+  for (int i = 0; i < NC_PER; ++i) {
+    const int c = min(c0 + i * stride, width - 1);
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) v.x[i][k] = x[(size_t)(r - min(k, inside)) * width + c];
+  }
+}
+
+template <typename T, int TAPS, int NC_PER>
+__device__ __forceinline__ void nc_load_rest(NormConvLoads<T, TAPS, NC_PER>& v, const T* __restrict__ st, const float* __restrict__ w,
+                                             const void* __restrict__ g, int g_bf16, int inside, int width, int c0,
+                                             int stride) {
   constexpr int KEEP = TAPS - 1;
-  __shared__ float red[4][TAPS];
+#pragma unroll
+  for (int i = 0; i < NC_PER; ++i) {
+    const int c = min(c0 + i * stride, width - 1);
+    v.g[i] = load_vec(g, g_bf16, c);
+#pragma unroll
+    for (int k = 1; k < TAPS; ++k)                    // place in the slot of the input k positions back
+      v.s[i][k] = st ? to_float(st[(size_t)min(max(KEEP - (k - inside), 0), KEEP - 1) * width + c]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) v.w[i][j] = w[(size_t)c * TAPS + j];
+  }
+}
+
+template <typename T, int TAPS, int NC_PER>
+__global__ __launch_bounds__(1024) void norm_conv_kernel(const float* __restrict__ x, const void* __restrict__ g,
+                                                         int g_bf16, float eps, const float* __restrict__ w,
+                                                         T* __restrict__ state, const int* __restrict__ row_req,
+                                                         const int* __restrict__ q_start,
+                                                         const int* __restrict__ req_rows, T* __restrict__ h,
+                                                         T* __restrict__ conv, int width, int own_state) {
+  constexpr int KEEP = TAPS - 1;
+  __shared__ float red[16][TAPS];
   __shared__ float s_inv[TAPS];
   const int r = blockIdx.x;
-  const int b = row_req[r];
-  const int first = q_start[b];
+  const int b = own_state ? r : row_req[r];
+  const int first = own_state ? r : q_start[b];
   const int inside = min(r - first, KEEP);            // rows of this request before r that the taps reach
   T* st = state && KEEP > 0 ? state + (size_t)req_rows[b] * KEEP * width : nullptr;
+  const int threads = blockDim.x, round = threads * NC_PER;
+  const bool one_round = width <= round;
+  NormConvLoads<T, TAPS, NC_PER> v;
   float ss[TAPS];
 #pragma unroll
   for (int k = 0; k < TAPS; ++k) ss[k] = 0.f;
-  for (int c = threadIdx.x; c < width; c += 256) {
-    float v[TAPS];
+  for (int c0 = threadIdx.x; c0 < width; c0 += round) {
+    nc_load_x<T, TAPS, NC_PER>(v, x, r, inside, width, c0, threads);
+    if (one_round) nc_load_rest<T, TAPS, NC_PER>(v, st, w, g, g_bf16, inside, width, c0, threads);
 #pragma unroll
-    for (int k = 0; k < TAPS; ++k) v[k] = x[(size_t)(r - min(k, inside)) * width + c];
+    for (int i = 0; i < NC_PER; ++i)
+      if (c0 + i * threads < width) {
 #pragma unroll
-    for (int k = 0; k < TAPS; ++k) ss[k] = fmaf(v[k], v[k], ss[k]);
+        for (int k = 0; k < TAPS; ++k) ss[k] = fmaf(v.x[i][k], v.x[i][k], ss[k]);
+      }
   }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = threads >> 6;
 #pragma unroll
   for (int k = 0; k < TAPS; ++k) ss[k] = wave_sum(ss[k]);
   if (lane == 0) {
@@ -202,38 +247,38 @@ __global__ __launch_bounds__(256) void norm_conv_kernel(const float* __restrict_
   }
   __syncthreads();
   if (threadIdx.x < TAPS) {
-    const float t = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+    float t = 0.f;
+    for (int i = 0; i < waves; ++i) t += red[i][threadIdx.x];
     s_inv[threadIdx.x] = 1.0f / sqrtf(t / (float)width + eps);
   }
   __syncthreads();
   float inv[TAPS];
 #pragma unroll
   for (int k = 0; k < TAPS; ++k) inv[k] = s_inv[k];
-  for (int c = threadIdx.x; c < width; c += 256) {
-    float xv[TAPS], sv[TAPS], wv[TAPS];
-    const float gc = load_vec(g, g_bf16, c);
-#pragma unroll
-    for (int k = 0; k < TAPS; ++k) xv[k] = x[(size_t)(r - min(k, inside)) * width + c];
-#pragma unroll
-    for (int k = 1; k < TAPS; ++k)                    // place in the slot of the input `k` positions back
-      sv[k] = st ? to_float(st[(size_t)min(max(KEEP - (k - inside), 0), KEEP - 1) * width + c]) : 0.f;
-#pragma unroll
-    for (int j = 0; j < TAPS; ++j) wv[j] = w[(size_t)c * TAPS + j];
-    const T own = from_float<T>(xv[0] * inv[0] * gc);
-    float acc = to_float(own);
-    acc = fmaf(wv[TAPS - 1], to_float(own), acc);
-    T hk[TAPS];
-    hk[0] = own;
-#pragma unroll
-    for (int k = 1; k < TAPS; ++k) {
-      hk[k] = k <= inside ? from_float<T>(xv[k] * inv[k] * gc) : from_float<T>(sv[k]);
-      acc = fmaf(wv[TAPS - 1 - k], to_float(hk[k]), acc);
+  for (int c0 = threadIdx.x; c0 < width; c0 += round) {
+    if (!one_round) {
+      nc_load_x<T, TAPS, NC_PER>(v, x, r, inside, width, c0, threads);
+      nc_load_rest<T, TAPS, NC_PER>(v, st, w, g, g_bf16, inside, width, c0, threads);
     }
-    h[(size_t)r * width + c] = own;
-    conv[(size_t)r * width + c] = from_float<T>(acc);
-    if (own_state && st) {
 #pragma unroll
-      for (int s = 0; s < KEEP; ++s) st[(size_t)s * width + c] = hk[KEEP - 1 - s];
+    for (int i = 0; i < NC_PER; ++i) {
+      const int c = c0 + i * threads;
+      if (c >= width) continue;
+      T hk[TAPS];
+      hk[0] = from_float<T>(v.x[i][0] * inv[0] * v.g[i]);
+      float acc = to_float(hk[0]);
+      acc = fmaf(v.w[i][TAPS - 1], to_float(hk[0]), acc);
+#pragma unroll
+      for (int k = 1; k < TAPS; ++k) {
+        hk[k] = k <= inside ? from_float<T>(v.x[i][k] * inv[k] * v.g[i]) : from_float<T>(v.s[i][k]);
+        acc = fmaf(v.w[i][TAPS - 1 - k], to_float(hk[k]), acc);
+      }
+      h[(size_t)r * width + c] = hk[0];
+      conv[(size_t)r * width + c] = from_float<T>(acc);
+      if (own_state && st) {
+#pragma unroll
+        for (int s = 0; s < KEEP; ++s) st[(size_t)s * width + c] = hk[KEEP - 1 - s];
+      }
     }
   }
 }
@@ -242,10 +287,24 @@ template <typename T>
 static void launch_norm_conv(int taps, int rows, hipStream_t stream, const float* x, const void* g, int g_bf16, float eps,
                              const float* w, T* state, const int* row_req, const int* q_start, const int* req_rows, T* h,
                              T* conv, int width, int own_state) {
-#define LLMLAB_NORM_CONV(N)                                                                                             \
-  case N:                                                                                                               \
-    hipLaunchKernelGGL((norm_conv_kernel<T, N>), dim3(rows), dim3(256), 0, stream, x, g, g_bf16, eps, w, state, row_req, \
-                       q_start, req_rows, h, conv, width, own_state);                                                   \
+  // few rows (a step bound by latency): a thread a channel up to a width of 1024, beyond that
+  // four channels a thread in blocks of 1024; many rows: blocks of 256, of which a compute unit
+  // holds several, four channels a thread
+  int threads = 256, per = 4;
+  if (rows <= 64 && width <= 1024) {
+    per = 1;
+    threads = (width + 63) / 64 * 64;
+  } else if (rows <= 64) {
+    while (threads < 1024 && threads * 4 < width) threads *= 2;
+  }
+#define LLMLAB_NORM_CONV(N)                                                                                               \
+  case N:                                                                                                                 \
+    if (per == 1)                                                                                                         \
+      hipLaunchKernelGGL((norm_conv_kernel<T, N, 1>), dim3(rows), dim3(threads), 0, stream, x, g, g_bf16, eps, w, state,   \
+                         row_req, q_start, req_rows, h, conv, width, own_state);                                          \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((norm_conv_kernel<T, N, 4>), dim3(rows), dim3(threads), 0, stream, x, g, g_bf16, eps, w, state,   \
+                         row_req, q_start, req_rows, h, conv, width, own_state);                                          \
     break;
   switch (taps) {
     LLMLAB_NORM_CONV(1) LLMLAB_NORM_CONV(2) LLMLAB_NORM_CONV(3) LLMLAB_NORM_CONV(4)
