@@ -218,7 +218,7 @@ def minodra_config(size):
         listed.append(dict(type="latent_attention", mixer=mixer, mlp=mlp))
     return lab.MinodraConfig.from_dict(dict(
         architecture="Minodra", vocab=DESIGN_VOCAB, width=width, norm=dict(eps=1e-6), layers=listed, canon=dict(taps=4),
-        embedding=dict(scale=12.0, bigram=dict(buckets=65521, mul_prev=127, mul_cur=7)), logit_softcap=30.0))
+        embedding=dict(scale=8.0, bigram=dict(buckets=65521, mul_prev=131, mul_cur=5)), logit_softcap=25.0))
 
 
 def minodra_flops(cfg, tokens):

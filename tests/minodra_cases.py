@@ -37,7 +37,7 @@ def moe(ff, experts, top, shared=None):
 #    expert chosen of nine; a large eps.
 CONFIGS = {
     "A": dict(architecture="Minodra", vocab=193, width=64, norm=dict(eps=1e-5), canon=dict(taps=4),
-              embedding=dict(scale=3.0, bigram=dict(buckets=61, mul_prev=127, mul_cur=7)), logit_softcap=5.0,
+              embedding=dict(scale=3.0, bigram=dict(buckets=61, mul_prev=113, mul_cur=11)), logit_softcap=5.0,
               layers=[latent(4, 16, 24, 24, 32, 0.5, mlp=dense(96)),
                       latent(2, 32, 16, 40, 20, 0.3, mlp=moe(24, 6, 3, shared=40)),
                       latent(3, 8, 8, 16, 96, 0.7, mlp=None)]),
@@ -46,7 +46,7 @@ CONFIGS = {
               layers=[latent(1, 40, 8, 12, 160, 0.25, mlp=moe(20, 3, 3)),
                       latent(6, 8, 16, 64, 8, 0.9, mlp=dense(52))]),
     "C": dict(architecture="Minodra", vocab=130, width=72, norm=dict(eps=1e-3), canon=dict(taps=1),
-              embedding=dict(scale=1.0), logit_softcap=30.0,
+              embedding=dict(scale=1.0), logit_softcap=20.0,
               layers=[latent(5, 24, 40, 48, 64, 0.35, mlp=moe(8, 9, 1, shared=64)),
                       latent(2, 64, 64, 32, 128, 0.2, mlp=dense(24)),
                       latent(4, 16, 16, 8, 33, 0.6, mlp=moe(16, 4, 2))]),

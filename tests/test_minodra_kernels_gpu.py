@@ -48,7 +48,7 @@ def on(device, *tensors):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hidden,vocab,buckets,norm", [(64, 50, 13, True), (100, 300, 1021, True), (24, 9, 1, False),
+@pytest.mark.parametrize("hidden,vocab,buckets,norm", [(64, 50, 13, True), (100, 300, 1019, True), (24, 9, 1, False),
                                                        (72, 40, 0, True)])
 def test_embed_pairs_over_steps(ops, emu, dtype, hidden, vocab, buckets, norm):
     """Three steps of three requests in slots 2, 0, 3: portions, single tokens, a request that starts
@@ -63,9 +63,9 @@ def test_embed_pairs_over_steps(ops, emu, dtype, hidden, vocab, buckets, norm):
         ids = torch.randint(0, vocab, (rows,), generator=g).int()
         desc = step_description(portions, starts, slots)
         want = torch.empty(rows, hidden)
-        emu.embed_pairs(table, pairs, ids, *desc, state_e if buckets else None, 3.5, buckets, 127, 7, weight, 1e-5, want)
+        emu.embed_pairs(table, pairs, ids, *desc, state_e if buckets else None, 3.5, buckets, 113, 11, weight, 1e-5, want)
         got = torch.empty(rows, hidden, device=DEV)
-        ops.embed_pairs(*on(DEV, table, pairs, ids, *desc), state_g if buckets else None, 3.5, buckets, 127, 7,
+        ops.embed_pairs(*on(DEV, table, pairs, ids, *desc), state_g if buckets else None, 3.5, buckets, 113, 11,
                         None if weight is None else weight.to(DEV), 1e-5, got)
         assert (got.cpu() - want).abs().max() <= 2e-5 * max(1.0, float(want.abs().max()))
         assert torch.equal(state_g.cpu(), state_e)
@@ -138,7 +138,7 @@ def test_norm_conv_over_steps(ops, emu, dtype, width, taps):
 
 
 @pytest.mark.parametrize("rows,width,cols,bias", [(1, 64, 64, True), (7, 100, 100, True), (5, 66, 1, False),
-                                                  (33, 320, 320, False), (3, 8, None, False)])
+                                                  (33, 328, 328, False), (3, 8, None, False)])
 def test_gated_add(ops, emu, rows, width, cols, bias):
     x, y = rnd((rows, width), torch.float32, 1), rnd((rows, width), torch.float32, 2)
     gate = rnd((rows, cols), torch.float32, 3, 2.0) if cols else None
@@ -153,11 +153,11 @@ def test_gated_add(ops, emu, rows, width, cols, bias):
 def test_softcap(ops, emu):
     x = rnd((5, 333), torch.float32, 1, 40.0)
     want = x.clone()
-    emu.softcap(want, 30.0)
+    emu.softcap(want, 25.0)
     got = x.to(DEV)
-    ops.softcap(got, 30.0)
+    ops.softcap(got, 25.0)
     assert (got.cpu() - want).abs().max() <= 1e-4
-    assert float(got.abs().max()) <= 30.0
+    assert float(got.abs().max()) <= 25.0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

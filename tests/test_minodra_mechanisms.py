@@ -82,7 +82,7 @@ def test_norm_with_one_number_as_its_weight(backend, dtype, hidden, eps):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("buckets,mul_prev,mul_cur", [(61, 127, 7), (1, 3, 5), (1021, 1, 1), (7, 1000003, 999983)])
+@pytest.mark.parametrize("buckets,mul_prev,mul_cur", [(61, 113, 11), (1, 3, 5), (1019, 1, 1), (7, 1000003, 999983)])
 def test_hashed_pairs_over_steps(backend, buckets, mul_prev, mul_cur):
     """Two sequences fed in unequal portions through slots 2 and 0; the previous token crosses every
     cut through the slot, and a sequence's first token takes the row behind the buckets."""
@@ -114,7 +114,7 @@ def test_hashed_pairs_over_steps(backend, buckets, mul_prev, mul_cur):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("cap", [30.0, 5.0, 0.7])
+@pytest.mark.parametrize("cap", [25.0, 5.0, 0.7])
 def test_soft_cap(backend, cap):
     ops = ops_of(backend)
     x = randn(7, 33, seed=3, scale=20.0)
@@ -188,7 +188,7 @@ def test_an_input_reaches_exactly_the_taps(backend, taps):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("rows,width", [(1, 8), (6, 72), (40, 320)])
+@pytest.mark.parametrize("rows,width", [(1, 8), (6, 72), (40, 328)])
 def test_gated_sum_into_the_stream(backend, rows, width):
     ops = ops_of(backend)
     x, y, h = randn(rows, width, seed=1), randn(rows, width, seed=2), randn(rows, width, seed=3)

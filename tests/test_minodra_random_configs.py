@@ -37,12 +37,12 @@ def draw_config(seed):
                                mlp=draw_mlp(rng)))
     raw = dict(architecture="Minodra", vocab=rng.choice([50, 131, 256]), width=rng.choice([32, 48, 64, 96, 128]),
                norm=dict(eps=rng.choice([1e-6, 1e-5, 1e-3])), canon=dict(taps=rng.choice([1, 2, 3, 4, 4, 5, 8])),
-               embedding=dict(scale=rng.choice([0.5, 1.0, 12.0])), layers=layers)
+               embedding=dict(scale=rng.choice([0.5, 1.0, 9.0])), layers=layers)
     if rng.random() < 0.75:
-        raw["embedding"]["bigram"] = dict(buckets=rng.choice([1, 2, 61, 1021, 4093]), mul_prev=rng.choice([1, 127, 65537]),
-                                          mul_cur=rng.choice([1, 7, 31]))
+        raw["embedding"]["bigram"] = dict(buckets=rng.choice([1, 2, 61, 1019, 4093]), mul_prev=rng.choice([1, 113, 65537]),
+                                          mul_cur=rng.choice([1, 11, 31]))
     if rng.random() < 0.6:
-        raw["logit_softcap"] = rng.choice([2.0, 10.0, 30.0])
+        raw["logit_softcap"] = rng.choice([2.0, 10.0, 25.0])
     return raw
 
 
@@ -79,7 +79,7 @@ def test_drawn_configuration(backend, seed):
 # over pages of 64.
 LARGER = {
     "X": dict(architecture="Minodra", vocab=701, width=384, norm=dict(eps=1e-6), canon=dict(taps=4),
-              embedding=dict(scale=12.0, bigram=dict(buckets=4093, mul_prev=127, mul_cur=7)), logit_softcap=30.0,
+              embedding=dict(scale=9.0, bigram=dict(buckets=4093, mul_prev=113, mul_cur=11)), logit_softcap=25.0,
               layers=[M.latent(6, 64, 64, 192, 128, 0.125, mlp=M.dense(1024)),
                       M.latent(12, 32, 48, 96, 256, 0.18, mlp=M.moe(96, 24, 6, shared=136)),
                       M.latent(3, 128, 64, 160, 64, 0.09, mlp=M.moe(104, 70, 3))]),
