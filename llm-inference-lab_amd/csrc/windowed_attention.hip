@@ -90,6 +90,8 @@ extern "C" int llmlab_project_norm_write(const float* proj, int ld, int rows, in
 
 static int g_force_plain = 0;      // tests and measurements: no matrix-core kernel
 extern "C" void llmlab_debug_windowed_attention_plain(int on) { g_force_plain = on; }
+static int g_private_tiles = 0;    // tests and measurements: prompts by the kernel whose waves fetch their own tiles
+extern "C" void llmlab_debug_windowed_attention_private_tiles(int on) { g_private_tiles = on; }
 
 // ------------------------------------------------------------------ attention
 // The query at position i of its request attends to the keys i - window < j <= i and to the
@@ -445,6 +447,203 @@ __global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(MfmaArg
   }
 }
 
+// Prompts whose heads read the same keys and values (one key/value head, or groups of a multiple
+// of four heads): a block takes 16 consecutive rows and FOUR heads, a wave a head.  The block
+// stages every tile of 32 keys and their values in LDS once (each thread asks for its 16-byte
+// pieces of the next tile before the products of this one and stores them after), and the waves
+// take their fragments from there instead of each from L2.  Key rows lie 16 bytes apart from a
+// multiple of 256 bytes and the values' quad rows 128, so that the lanes of a read spread over the
+// banks.  Everything else (the list of tiles, masks, the running softmax, the transposed
+// products) is the kernel's above; all waves of a block walk the same tiles, so the barriers
+// are reached by all.
+template <int DC, int EB>
+__global__ __launch_bounds__(256) void sink_window_attention_shared_kernel(MfmaArgs a) {
+  constexpr int D = 32 * DC, E = 16 * EB;
+  constexpr int KROW = D + 8, VROW = 4 * E + 64;
+  constexpr int KCHUNKS = 4 * D, VCHUNKS = 4 * E;            // 16-byte pieces of a tile's keys / values
+  constexpr int KCH = (KCHUNKS + 255) / 256, VCH = (VCHUNKS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) bf16_t ks[2 * 16 * KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t vs[2 * 4 * VROW];
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, g4 = lane >> 4, wave = tid >> 6;
+  const int r0 = blockIdx.x * 16;
+  if (r0 >= a.n_rows) return;
+  const int h_raw = blockIdx.y * 4 + wave;
+  const bool head_ok = h_raw < a.n_heads;
+  const int h = head_ok ? h_raw : a.n_heads - 1;
+  const int g = (blockIdx.y * 4) / (a.n_heads / a.n_kv);
+  const int r = r0 + c;
+  const bool row_ok = r < a.n_rows;
+  const int pos = row_ok ? a.positions[r] : 0;
+  const int req = row_ok ? a.row_req[r] : -1;
+  bf16x8 zero8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) zero8[i] = (bf16_t)0.f;
+  bf16x8 qf[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc)
+    qf[dc] = row_ok ? *(const bf16x8*)(a.q + ((size_t)r * a.n_heads + h) * D + 32 * dc + 8 * g4) : zero8;
+  Running<EB> run;
+  run.m = a.sink ? a.sink[h] : NEG_INF;
+  run.l = a.sink ? 1.f : 0.f;
+#pragma unroll
+  for (int eb = 0; eb < EB; ++eb) run.o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int b_first = __builtin_amdgcn_readfirstlane(a.row_req[r0]);
+  const int b_last = __builtin_amdgcn_readfirstlane(a.row_req[(r0 + 15 < a.n_rows ? r0 + 15 : a.n_rows - 1)]);
+  for (int b = b_first; b <= b_last; ++b) {
+    if (a.long_from > 0 && a.q_start[b + 1] - a.q_start[b] < a.long_from) continue;      // (the other kernels' rows)
+    const bool mine = req == b;
+    int p_lo = mine ? pos : 0x7fffffff, p_hi = mine ? pos : -1;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      p_lo = min(p_lo, __shfl_xor(p_lo, off, WAVE));
+      p_hi = max(p_hi, __shfl_xor(p_hi, off, WAVE));
+    }
+    if (p_hi < 0) continue;
+    const KeyTiles kt(p_lo, p_hi, a.window, a.keep_first);
+    const int* pages = a.table + (size_t)b * a.max_pages;
+    bf16x8 kreg[KCH], vreg[VCH];
+    // the 16-byte pieces of tile t that this thread brings
+    auto fetch = [&](int t) {
+      const int j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
+      const int end = t < kt.tiles_a ? kt.a_end : kt.end_b;
+      size_t kbase[2], vbase[2];
+      bool have[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int ju = j0 + 16 * u;
+        have[u] = ju < end;
+        kbase[u] = vbase[u] = 0;
+        if (have[u]) {
+          const int page = pages[ju / a.page_size];
+          const size_t head = ((size_t)page * a.n_kv + g) * a.page_size;
+          const int off = ju % a.page_size;
+          kbase[u] = (head + off) * D;
+          vbase[u] = head * E + (size_t)(off >> 2) * E * 4;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < KCH; ++i) {
+        const int idx = tid + 256 * i;
+        const int u = idx / (2 * D), rem = idx % (2 * D);
+        kreg[i] = (idx < KCHUNKS && have[u & 1]) ? *(const bf16x8*)(a.k_cache + kbase[u & 1] + (size_t)rem * 8) : zero8;
+      }
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int idx = tid + 256 * i;
+        const int u = idx / (2 * E), rem = idx % (2 * E);
+        vreg[i] = (idx < VCHUNKS && have[u & 1]) ? *(const bf16x8*)(a.v_cache + vbase[u & 1] + (size_t)rem * 8) : zero8;
+      }
+    };
+    auto stash = [&]() {
+#pragma unroll
+      for (int i = 0; i < KCH; ++i) {
+        const int idx = tid + 256 * i;
+        if (idx < KCHUNKS) {
+          const int u = idx / (2 * D), rem = idx % (2 * D);
+          const int key = rem / (D / 8), part = rem % (D / 8);
+          *(bf16x8*)(ks + (u * 16 + key) * KROW + part * 8) = kreg[i];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < VCH; ++i) {
+        const int idx = tid + 256 * i;
+        if (idx < VCHUNKS) {
+          const int u = idx / (2 * E), rem = idx % (2 * E);
+          const int quad = rem / (E / 2), within = rem % (E / 2);
+          *(bf16x8*)(vs + (u * 4 + quad) * VROW + within * 8) = vreg[i];
+        }
+      }
+    };
+    __syncthreads();                                  // (the request before this one has been read)
+    fetch(0);
+    stash();
+    __syncthreads();
+    for (int t = 0; t < kt.tiles; ++t) {
+      if (t + 1 < kt.tiles) fetch(t + 1);
+      const int j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
+      const int end = t < kt.tiles_a ? kt.a_end : kt.end_b;
+      const bool have1 = j0 + 16 < end;
+      floatx4 s[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        s[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+          const bf16x8 kf = *(const bf16x8*)(ks + (u * 16 + c) * KROW + 32 * dc + 8 * g4);
+          s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[dc], s[u], 0, 0, 0);
+        }
+      }
+      float tmax = NEG_INF;
+      const bool interior = have1 && j0 + 31 < end && j0 + 31 <= kt.p_lo &&
+                            (a.window <= 0 || kt.p_hi - j0 < a.window || j0 + 31 < a.keep_first);
+      if (interior) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            s[u][i] = mine ? s[u][i] * a.scale : NEG_INF;
+            tmax = fmaxf(tmax, s[u][i]);
+          }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int j = j0 + 16 * u + 4 * g4 + i;
+            const bool ok = mine && j < end && sees(pos, j, a.window, a.keep_first);
+            s[u][i] = ok ? s[u][i] * a.scale : NEG_INF;
+            tmax = fmaxf(tmax, s[u][i]);
+          }
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+      const float m_new = fmaxf(run.m, tmax);
+      const float m_use = m_new == NEG_INF ? 0.f : m_new;
+      const float corr = run.m == NEG_INF ? 0.f : __expf(run.m - m_use);
+      float sum = 0.f;
+      bf16x8 pf;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = __expf(s[u][i] - m_use);       // (exp(-inf) = 0 for a masked key)
+          sum += p;
+          pf[4 * u + i] = (bf16_t)p;
+        }
+      sum += __shfl_xor(sum, 16, WAVE);
+      sum += __shfl_xor(sum, 32, WAVE);
+      run.l = run.l * corr + sum;
+      run.m = m_new;
+#pragma unroll
+      for (int eb = 0; eb < EB; ++eb) {
+        bf16x8 vf;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const bf16x4 quad = *(const bf16x4*)(vs + (u * 4 + g4) * VROW + (16 * eb + c) * 4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) vf[4 * u + i] = quad[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) run.o[eb][i] *= corr;
+        run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, run.o[eb], 0, 0, 0);
+      }
+      __syncthreads();                                // (every wave has read the tile)
+      if (t + 1 < kt.tiles) stash();
+      __syncthreads();
+    }
+  }
+  if (!row_ok || !head_ok) return;
+  if (a.long_from > 0 && a.q_start[req + 1] - a.q_start[req] < a.long_from) return;
+  const float inv = 1.0f / run.l;
+#pragma unroll
+  for (int eb = 0; eb < EB; ++eb) {
+    bf16x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (bf16_t)(run.o[eb][i] * inv);
+    *(bf16x4*)(a.out + ((size_t)r * a.n_heads + h) * E + 16 * eb + 4 * g4) = w;
+  }
+}
+
 // Decoding (requests that bring fewer than long_from rows): a wave takes ONE row, the heads of
 // one key/value head (16 at a time) and one of `splits` shares of the row's key tiles, so that
 // few rows still fill the chip.  With one share the result is final; else the share's
@@ -569,6 +768,7 @@ static void launch_mfma(int EBv, int which, dim3 grid, dim3 block, hipStream_t s
 #define LLMLAB_MFMA(EBC)                                                                                      \
   case EBC:                                                                                                   \
     if (which == 0) hipLaunchKernelGGL((sink_window_attention_mfma_kernel<DC, EBC>), grid, block, 0, stream, a); \
+    else if (which == 2) hipLaunchKernelGGL((sink_window_attention_shared_kernel<DC, EBC>), grid, block, 0, stream, a); \
     else hipLaunchKernelGGL((sink_window_attention_grouped_kernel<DC, EBC>), grid, block, 0, stream, a);      \
     break;
   switch (EBv) {
@@ -581,6 +781,7 @@ static void launch_mfma_any(int D, int E, int which, dim3 grid, dim3 block, hipS
 #define LLMLAB_MFMA_SQUARE(DCV)                                                                                          \
   case DCV:                                                                                                             \
     if (which == 0) hipLaunchKernelGGL((sink_window_attention_mfma_kernel<DCV, 2 * DCV>), grid, block, 0, stream, a);     \
+    else if (which == 2) hipLaunchKernelGGL((sink_window_attention_shared_kernel<DCV, 2 * DCV>), grid, block, 0, stream, a); \
     else hipLaunchKernelGGL((sink_window_attention_grouped_kernel<DCV, 2 * DCV>), grid, block, 0, stream, a);            \
     return;
   if (D > 128) {
@@ -627,7 +828,12 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
                page_size, positions, row_req, window, keep_first, sink, scale, (bf16_t*)out, q_start, long_from, 1,
                nullptr, nullptr};
     if (launches & 2) {
-      launch_mfma_any(D, E, 0, dim3((rows + 63) / 64, n_heads), dim3(256), stream, a);
+      // heads that read the same keys and values share the tiles a block stages in LDS
+      const int group = n_heads / n_kv;
+      if (!g_private_tiles && group >= 3 && (n_kv == 1 || group % 4 == 0))
+        launch_mfma_any(D, E, 2, dim3((rows + 15) / 16, (n_heads + 3) / 4), dim3(256), stream, a);
+      else
+        launch_mfma_any(D, E, 0, dim3((rows + 63) / 64, n_heads), dim3(256), stream, a);
       LLMLAB_LAUNCH_CHECK("sink_window_attention (prompts)");
     }
     if (launches & 1) {

@@ -1061,6 +1061,8 @@ class HipOps:
                 lib.llmlab_sink_window_attention_has_mfma.restype = _c_int
                 lib.llmlab_debug_windowed_attention_plain.argtypes = [_c_int]
                 lib.llmlab_debug_windowed_attention_plain.restype = None
+                lib.llmlab_debug_windowed_attention_private_tiles.argtypes = [_c_int]
+                lib.llmlab_debug_windowed_attention_private_tiles.restype = None
                 lib.llmlab_latent_norm_write.argtypes = [
                     _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr,
                     _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
@@ -1357,6 +1359,12 @@ class HipOps:
     def force_plain_windowed_attention(self, on: bool) -> None:
         """Tests and measurements: no matrix-core kernel for the windowed attention."""
         self._mixer_lib("windowed_attention").llmlab_debug_windowed_attention_plain(1 if on else 0)
+        self.debug_epoch += 1
+
+    def force_private_attention_tiles(self, on: bool) -> None:
+        """Tests and measurements: prompts of heads that read the same keys and values go to the
+        kernel whose waves fetch their own tiles, not to the one that stages them in LDS for a block."""
+        self._mixer_lib("windowed_attention").llmlab_debug_windowed_attention_private_tiles(1 if on else 0)
         self.debug_epoch += 1
 
     def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,

@@ -226,7 +226,7 @@ def test_sigmoid_router_choice(ops, emu, rows, outputs, top):
 
 
 @pytest.mark.parametrize("latent", [32, 96, 160, 256])
-@pytest.mark.parametrize("heads", [3, 16, 20])
+@pytest.mark.parametrize("heads", [3, 6, 16, 21])
 def test_attention_over_one_cached_vector_per_token(ops, emu, latent, heads):
     """The attention kernels in the latent form (one key/value head, values = keys, a sink): a portion
     of a prompt behind a history, a whole prompt and two decoding requests in one step, by the
@@ -245,8 +245,10 @@ def test_attention_over_one_cached_vector_per_token(ops, emu, latent, heads):
     want = torch.zeros(rows, heads * latent, dtype=dtype)
     emu.sink_window_attention(q, heads, 1, latent, latent, k_cache, v_cache, table, page, positions, row_req, None, 0,
                               sink, 0.7, want)
-    for plain in (False, True):
+    # (prompts' tiles staged in LDS for a block of four heads; fetched by every wave for itself; no matrix cores)
+    for plain, private in ((False, False), (False, True), (True, False)):
         ops.force_plain_windowed_attention(plain)
+        ops.force_private_attention_tiles(private)
         try:
             long_from = ops.windowed_attention_long_rows(dtype, latent, latent, page)
             assert bool(long_from) == (not plain)
@@ -256,4 +258,5 @@ def test_attention_over_one_cached_vector_per_token(ops, emu, latent, heads):
                                       q_start.to(DEV), long_from, 3, 200)
         finally:
             ops.force_plain_windowed_attention(False)
-        assert (got.cpu().float() - want.float()).abs().max() <= 2e-2, (latent, heads, plain)
+            ops.force_private_attention_tiles(False)
+        assert (got.cpu().float() - want.float()).abs().max() <= 2e-2, (latent, heads, plain, private)
