@@ -457,7 +457,7 @@ __global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(MfmaArg
 // products) is the kernel's above; all waves of a block walk the same tiles, so the barriers
 // are reached by all.
 template <int DC, int EB>
-__global__ __launch_bounds__(256) void sink_window_attention_shared_kernel(MfmaArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void sink_window_attention_shared_kernel(MfmaArgs a) {
   constexpr int D = 32 * DC, E = 16 * EB;
   constexpr int KROW = D + 8, VROW = 4 * E + 64;
   constexpr int KCHUNKS = 4 * D, VCHUNKS = 4 * E;            // 16-byte pieces of a tile's keys / values
