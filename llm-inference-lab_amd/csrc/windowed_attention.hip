@@ -109,7 +109,7 @@ __device__ __forceinline__ bool sees(int i, int j, int window, int keep_first) {
 // ---- plain kernel: one wave per (row, head); float32 products.  Keys are taken 64 at a
 // time: lane n scores one key (its own row of D numbers), the weights go through LDS, then
 // lane e sums the values' channel e (and e + 64, ...) a quad of keys a load.
-constexpr int MAX_E_PER_LANE = 4;      // value width up to 256
+constexpr int MAX_E_PER_LANE = 16;     // value width up to 1024
 
 template <typename T>
 __device__ __forceinline__ float dot_row(const float* __restrict__ q, const T* __restrict__ k, int D);

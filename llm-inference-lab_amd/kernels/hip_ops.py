@@ -1289,8 +1289,8 @@ class HipOps:
     def check_windowed_attention_sizes(self, num_heads, num_kv_heads, key_dim, value_dim, dtype) -> None:
         if num_heads % num_kv_heads:
             raise UnsupportedSizeError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
-        if not 0 < value_dim <= 256 or not 0 < key_dim <= 4096:
-            raise UnsupportedSizeError(f"windowed attention takes keys up to 4096 and values up to 256 wide, "
+        if not 0 < value_dim <= 1024 or not 0 < key_dim <= 4096:
+            raise UnsupportedSizeError(f"windowed attention takes keys up to 4096 and values up to 1024 wide, "
                                        f"got {key_dim} and {value_dim}")
         self._mixer_lib("windowed_attention")
 
@@ -1401,8 +1401,8 @@ class HipOps:
             self._need(sink, "sink", torch.float32)
             if sink.numel() != num_heads:
                 raise ValueError("windowed attention: one sink per head")
-        if value_dim > 256:
-            raise UnsupportedSizeError(f"windowed attention takes values up to 256 wide, got {value_dim}")
+        if value_dim > 1024:
+            raise UnsupportedSizeError(f"windowed attention takes values up to 1024 wide, got {value_dim}")
         self._call(lib.llmlab_sink_window_attention, self._ptr(q), _dt(q), rows, num_heads, num_kv_heads, key_dim,
                    value_dim, self._ptr(k_cache), self._ptr(v_cache), self._ptr(block_table), block_table.stride(0),
                    page_size, self._ptr(positions), self._ptr(row_req), int(window) if window else 0,

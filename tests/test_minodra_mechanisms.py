@@ -149,7 +149,7 @@ def conv_over_cuts(ops, dtype, h, weight, cuts, fused, norm_w=None, eps=1e-5):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps", [1, 2, 4, 7])
+@pytest.mark.parametrize("taps", [1, 2, 4, 7, 11])
 @pytest.mark.parametrize("cuts", [[23], [1] * 23, [2, 2, 3, 1, 9, 2, 4], [5, 18]])
 def test_convolution_over_cuts(backend, dtype, taps, cuts):
     """``h + conv(h)`` of a sequence cut into portions (shorter than the taps, single tokens, whole)
@@ -355,7 +355,8 @@ def test_a_key_anywhere_in_the_past_is_seen(backend, decoded):
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("decoded", [False, True])
 @pytest.mark.parametrize("sizes", [dict(heads=4, dim=32, vdim=16, q_rank=48, kv_rank=64),
-                                   dict(heads=2, dim=8, vdim=24, q_rank=8, kv_rank=136)])
+                                   dict(heads=2, dim=8, vdim=24, q_rank=8, kv_rank=136),
+                                   dict(heads=3, dim=16, vdim=16, q_rank=24, kv_rank=300)])
 def test_a_far_key_among_hundreds(backend, decoded, sizes):
     raw, tensors = one_layer_with_a_key_that_stands_out(**sizes)
     for back in (250, 329):

@@ -1,6 +1,6 @@
 """Minodra configurations drawn at random (widths, head counts and key / value sizes beside the
-multiples of 16, latents narrower and wider than a head and beside the multiples of 32, one to eight
-taps, pair tables of one bucket to thousands or none, with and without a soft cap, dense feed-forwards,
+multiples of 16, latents narrower and wider than a head, beside the multiples of 32 and up to 520, one to
+twelve taps, pair tables of one bucket to thousands or none, with and without a soft cap, dense feed-forwards,
 mixtures with every expert chosen or one, with and without a shared expert, layers without a
 feed-forward): mixed batches through the engine against the plain implementation, float32 tight and
 bfloat16 position by position."""
@@ -33,10 +33,10 @@ def draw_config(seed):
     for _ in range(rng.randint(1, 4)):
         layers.append(M.latent(rng.choice([1, 2, 3, 5, 8]), rng.choice([8, 16, 24, 32, 40, 64]),
                                rng.choice([8, 16, 24, 48, 64]), rng.choice([8, 12, 24, 64, 100]),
-                               rng.choice([8, 20, 32, 33, 64, 96, 128, 136, 200]), rng.choice([0.05, 0.2, 0.5, 1.0]),
+                               rng.choice([8, 20, 32, 33, 64, 96, 128, 136, 200, 300, 520]), rng.choice([0.05, 0.2, 0.5, 1.0]),
                                mlp=draw_mlp(rng)))
     raw = dict(architecture="Minodra", vocab=rng.choice([50, 131, 256]), width=rng.choice([32, 48, 64, 96, 128]),
-               norm=dict(eps=rng.choice([1e-6, 1e-5, 1e-3])), canon=dict(taps=rng.choice([1, 2, 3, 4, 4, 5, 8])),
+               norm=dict(eps=rng.choice([1e-6, 1e-5, 1e-3])), canon=dict(taps=rng.choice([1, 2, 3, 4, 4, 5, 8, 9, 12])),
                embedding=dict(scale=rng.choice([0.5, 1.0, 9.0])), layers=layers)
     if rng.random() < 0.75:
         raw["embedding"]["bigram"] = dict(buckets=rng.choice([1, 2, 61, 1019, 4093]), mul_prev=rng.choice([1, 113, 65537]),
