@@ -51,6 +51,7 @@ class LatentAttention(Mixer):
         self.head_dim, self.value_dim = int(head_dim), int(value_dim)
         self.q_rank, self.kv_rank = int(q_rank), int(kv_rank)
         self.q_rank_laid = (self.q_rank + 7) // 8 * 8                   # inner sizes of products: multiples of 8
+        self.value_laid = (self.value_dim + 7) // 8 * 8                 # (zero rows of V_a, zero columns of W_o behind a head)
         self.latent = (self.kv_rank + LATENT_PAD - 1) // LATENT_PAD * LATENT_PAD
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.has_sink, self.output_gate = bool(sink), output_gate
@@ -81,7 +82,7 @@ class LatentAttention(Mixer):
         super().bind(tensors, ops, dtype)
         ops.check_windowed_attention_sizes(self.num_heads, 1, self.latent, self.latent, dtype)
         ops.check_product_sizes(self.hidden_size, dtype, "attention projections (hidden size)")
-        ops.check_product_sizes(self.num_heads * self.value_dim, dtype, "attention output projection (heads * value size)")
+        ops.check_product_sizes(self.num_heads * self.value_laid, dtype, "attention output projection (heads * value size)")
         t, a = self.tensor_names, self.num_heads
 
         def grown(x, rows=None, columns=None):
@@ -103,8 +104,12 @@ class LatentAttention(Mixer):
         # head a's query in the latent's coordinates: U_a^T q_a, a product with U_a^T [latent, dim]
         uk = grown(tensors[t["uk_weight"]], columns=self.latent).view(a, self.head_dim, self.latent)
         self.w_absorb = uk.transpose(1, 2).contiguous()                                   # [heads, latent, dim]
-        self.w_value = grown(tensors[t["uv_weight"]], columns=self.latent).view(a, self.value_dim, self.latent).contiguous()
-        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
+        uv, wo = tensors[t["uv_weight"]], tensors[t["o_weight"]]
+        self.w_value = torch.zeros((a, self.value_laid, self.latent), dtype=uv.dtype, device=uv.device)
+        self.w_value[:, :self.value_dim, :self.kv_rank] = uv.view(a, self.value_dim, self.kv_rank)
+        o_laid = torch.zeros((self.hidden_size, a, self.value_laid), dtype=wo.dtype, device=wo.device)
+        o_laid[:, :, :self.value_dim] = wo.view(self.hidden_size, a, self.value_dim)
+        self.w_o = ops.prepare_weight(o_laid.view(self.hidden_size, a * self.value_laid).contiguous())
         if self.has_sink:
             self.sink = tensors[t["sink"]].float().contiguous()
 
@@ -138,7 +143,7 @@ class LatentAttention(Mixer):
             live(attend)
         else:
             attend()
-        heads = ctx.scratch("latent_attention.heads", (rows, a * self.value_dim), self.dtype)
+        heads = ctx.scratch("latent_attention.heads", (rows, a * self.value_laid), self.dtype)
         ops.head_products(mixed, self.w_value, heads, gate)       # (the heads' sigmoid gates ride on the product)
         ops.linear_logits(heads, self.w_o, out)
 

@@ -356,7 +356,8 @@ def test_a_key_anywhere_in_the_past_is_seen(backend, decoded):
 @pytest.mark.parametrize("decoded", [False, True])
 @pytest.mark.parametrize("sizes", [dict(heads=4, dim=32, vdim=16, q_rank=48, kv_rank=64),
                                    dict(heads=2, dim=8, vdim=24, q_rank=8, kv_rank=136),
-                                   dict(heads=3, dim=16, vdim=16, q_rank=24, kv_rank=300)])
+                                   dict(heads=3, dim=16, vdim=16, q_rank=24, kv_rank=300),
+                                   dict(heads=5, dim=12, vdim=12, q_rank=20, kv_rank=40)])
 def test_a_far_key_among_hundreds(backend, decoded, sizes):
     raw, tensors = one_layer_with_a_key_that_stands_out(**sizes)
     for back in (250, 329):
