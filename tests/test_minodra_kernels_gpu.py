@@ -97,7 +97,7 @@ def test_causal_conv_over_steps(ops, emu, dtype, width, taps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width,taps", [(64, 4), (100, 2), (24, 7), (40, 1), (896, 4), (72, 8)])
+@pytest.mark.parametrize("width,taps", [(64, 4), (100, 2), (24, 7), (40, 1), (896, 4), (72, 8), (2500, 4), (5000, 3)])
 def test_norm_conv_over_steps(ops, emu, dtype, width, taps):
     """The norm of the stream's rows and the convolution over them in one launch: portions shorter
     and longer than the taps, single tokens, a sequence's start inside a step, steps in which every
