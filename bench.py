@@ -228,8 +228,11 @@ def minodra_flops(cfg, tokens):
     w, total = cfg.width, 0
     pairs = tokens * (tokens + 1) // 2
     for l in cfg.layers:
-        total += tokens * 2 * (w * (l.q_rank + l.kv_rank + l.heads) + l.q_rank * l.heads * l.dim
-                               + l.heads * l.kv_rank * (l.dim + l.vdim) + l.heads * l.vdim * w + w * w)
+        latent = (l.kv_rank + 31) // 32 * 32
+        to_latent = (l.q_rank * l.heads * l.kv_rank if latent <= 2 * l.dim      # (one matrix, made when the mixer is bound)
+                     else l.q_rank * l.heads * l.dim + l.heads * l.kv_rank * l.dim)
+        total += tokens * 2 * (w * (l.q_rank + l.kv_rank + l.heads) + to_latent
+                               + l.heads * l.kv_rank * l.vdim + l.heads * l.vdim * w + w * w)
         total += 4 * pairs * l.heads * l.kv_rank
         f = l.mlp
         if f is not None and f.kind == "dense":

@@ -34,16 +34,23 @@ class LatentAttention(Mixer):
     portions.  The pages hold the vector twice, row by row for the scores and in quads of keys
     for the weighted sum (the two orders the attention kernels read).
 
+    ``fold_query``: ``U_a^T q_a = (U_a^T W_uq,a) c_q``, so the two products that take the query's
+    latent to the cached vector's coordinates can be ONE matrix ``[heads * latent, q_rank]``, made
+    in float32 when the part is bound and rounded once.  It has ``latent / dim`` times the rows of
+    ``W_uq`` and saves a launch and the head-sized queries' trip through memory; None: folded
+    when the latent is at most ``FOLD_UP_TO`` times a head's size.
+
     Tensor roles: ``dq_weight, dq_norm, uq_weight, dkv_weight, dkv_norm, uk_weight, uv_weight,
     sink, gate_weight, o_weight``."""
 
     writes_output = True
     keeps_launches = True      # (what depends on the step beyond its rows is asked for at the launch)
     OUTPUT_GATES = (None, "sigmoid")
+    FOLD_UP_TO = 2
 
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, q_rank: int, kv_rank: int,
                  scale: float, tensors: Dict[str, str], norm_eps: float = 1e-6, sink: bool = True,
-                 output_gate: str = "sigmoid"):
+                 output_gate: str = "sigmoid", fold_query: bool = None):
         super().__init__(tensors)
         if output_gate not in self.OUTPUT_GATES:
             raise ValueError(f"an output gate is one of {self.OUTPUT_GATES}, got {output_gate!r}")
@@ -55,6 +62,7 @@ class LatentAttention(Mixer):
         self.latent = (self.kv_rank + LATENT_PAD - 1) // LATENT_PAD * LATENT_PAD
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.has_sink, self.output_gate = bool(sink), output_gate
+        self.fold_query = self.latent <= self.FOLD_UP_TO * self.head_dim if fold_query is None else bool(fold_query)
         self.w_in = self.w_uq = self.w_absorb = self.w_value = self.w_o = None
         self.q_norm = self.c_norm = self.sink = None
 
@@ -98,12 +106,18 @@ class LatentAttention(Mixer):
         if self.output_gate:
             rows.append(tensors[t["gate_weight"]])
         self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())
-        self.w_uq = ops.prepare_weight(grown(tensors[t["uq_weight"]], columns=self.q_rank_laid).contiguous())
+        uq = grown(tensors[t["uq_weight"]], columns=self.q_rank_laid)
         self.q_norm = grown(tensors[t["dq_norm"]].float().view(1, -1), columns=self.q_rank_laid).view(-1).contiguous()
         self.c_norm = grown(tensors[t["dkv_norm"]].float().view(1, -1), columns=self.latent).view(-1).contiguous()
         # head a's query in the latent's coordinates: U_a^T q_a, a product with U_a^T [latent, dim]
         uk = grown(tensors[t["uk_weight"]], columns=self.latent).view(a, self.head_dim, self.latent)
-        self.w_absorb = uk.transpose(1, 2).contiguous()                                   # [heads, latent, dim]
+        if self.fold_query:
+            folded = torch.bmm(uk.float().transpose(1, 2), uq.float().view(a, self.head_dim, self.q_rank_laid))
+            self.w_uq = ops.prepare_weight(folded.reshape(a * self.latent, self.q_rank_laid).to(uq.dtype).contiguous())
+            self.w_absorb = None
+        else:
+            self.w_uq = ops.prepare_weight(uq.contiguous())
+            self.w_absorb = uk.transpose(1, 2).contiguous()                               # [heads, latent, dim]
         uv, wo = tensors[t["uv_weight"]], tensors[t["o_weight"]]
         self.w_value = torch.zeros((a, self.value_laid, self.latent), dtype=uv.dtype, device=uv.device)
         self.w_value[:, :self.value_dim, :self.kv_rank] = uv.view(a, self.value_dim, self.kv_rank)
@@ -126,10 +140,13 @@ class LatentAttention(Mixer):
         ops.latent_norm_write(proj, self.q_rank, self.q_rank_laid, self.kv_rank, self.latent, self.gates, self.q_norm,
                               self.c_norm, self.norm_eps, cq, gate, entry.k_cache, entry.v_cache, group.page_size,
                               ctx.positions, ctx.row_req, group.block_table)
-        q = ctx.scratch("latent_attention.q", (rows, a * self.head_dim), self.dtype)
-        ops.linear(cq, self.w_uq, q)
         ql = ctx.scratch("latent_attention.q_in_latent", (rows, a * self.latent), self.dtype)
-        ops.head_products(q, self.w_absorb, ql)
+        if self.fold_query:
+            ops.linear(cq, self.w_uq, ql)
+        else:
+            q = ctx.scratch("latent_attention.q", (rows, a * self.head_dim), self.dtype)
+            ops.linear(cq, self.w_uq, q)
+            ops.head_products(q, self.w_absorb, ql)
         mixed = ctx.scratch("latent_attention.mixed", (rows, a * self.latent), self.dtype)
 
         def attend():

@@ -418,3 +418,24 @@ def test_the_gate_of_a_head_reads_the_mixers_input(backend):
         got = run_prompt_or_decode(raw, tensors, ids, backend, decode_from)
         assert float((got - want).abs().max()) < 2e-4
     assert math.isfinite(float(want.abs().max()))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("fold", [0, 100])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_the_querys_two_products_as_one_matrix_or_apart(backend, fold, name, monkeypatch):
+    """``U_a^T (W_uq c_q)`` in two products, or ``(U_a^T W_uq) c_q`` with one matrix made when the part
+    is bound: the same logits, in every layer of a configuration whatever its sizes would choose."""
+    from llm_inference_lab_amd.parts.latent_attention import LatentAttention
+    monkeypatch.setattr(LatentAttention, "FOLD_UP_TO", fold)
+    cfg = M.config_of(name)
+    ids = M.random_ids(cfg, 41, 3)
+    want = M.plain_logits(name, 1, ids)
+    kw = dict(ops=EmuOps(), device="cpu") if backend == "emu" else {}
+    engine = M.make_engine(name, 1, "f32", **kw)
+    assert all(b.mixer.fold_query == (fold > 0) for b in engine.model.blocks)
+    req = engine.open("r")
+    first = engine.step([H.lab.StepEntry(req, ids[:30], list(range(30)))]).float().cpu().double()
+    rest = [engine.step([H.lab.StepEntry(req, [t], [0])]).float().cpu().double()[0] for t in ids[30:]]
+    got = torch.cat([first, torch.stack(rest)])
+    assert float((got - want).abs().max()) < 2e-4
