@@ -340,12 +340,16 @@ extern "C" int llmlab_norm_conv(const float* x, const void* g, int g_dtype, floa
 
 // ------------------------------------------------------------------ gated sum into the stream
 // x[r, c] += y[r, c] * sigmoid(gate[r, c or 0] + bias[c]); gate null: x += y.  All float32.
-__global__ void gated_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ gate,
-                                 int gate_cols, const float* __restrict__ bias, int width, size_t n) {
+// y may come in `pieces` (a product left cut along its inner size): y = sum_s y[s * piece_stride + .],
+// summed in the pieces' order.
+__global__ void gated_add_kernel(float* __restrict__ x, const float* __restrict__ y, int pieces, size_t piece_stride,
+                                 const float* __restrict__ gate, int gate_cols, const float* __restrict__ bias, int width,
+                                 size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     const size_t r = i / width;
     const int c = (int)(i - r * width);
     float v = y[i];
+    for (int s = 1; s < pieces; ++s) v += y[s * piece_stride + i];
     if (gate) {
       float g = gate_cols == 1 ? gate[r] : gate[i];
       if (bias) g += bias[c];
@@ -355,12 +359,20 @@ __global__ void gated_add_kernel(float* __restrict__ x, const float* __restrict_
   }
 }
 
-__global__ void gated_add4_kernel(floatx4* __restrict__ x, const floatx4* __restrict__ y, const floatx4* __restrict__ gate,
-                                  const floatx4* __restrict__ bias, int width4, size_t n4) {
+constexpr int GATED_ADD_MAX_PIECES = 8;
+__global__ void gated_add4_kernel(floatx4* __restrict__ x, const floatx4* __restrict__ y, int pieces, size_t piece_stride4,
+                                  const floatx4* __restrict__ gate, const floatx4* __restrict__ bias, int width4,
+                                  size_t n4) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
     floatx4 g = gate[i];
     if (bias) g += bias[i % width4];
-    const floatx4 v = y[i];
+    floatx4 part[GATED_ADD_MAX_PIECES];            // (the pieces' loads together; past the last: the last again, dropped)
+#pragma unroll
+    for (int s = 0; s < GATED_ADD_MAX_PIECES; ++s) part[s] = y[(size_t)min(s, pieces - 1) * piece_stride4 + i];
+    floatx4 v = part[0];
+#pragma unroll
+    for (int s = 1; s < GATED_ADD_MAX_PIECES; ++s)
+      if (s < pieces) v += part[s];
     floatx4 o = x[i];
 #pragma unroll
     for (int q = 0; q < 4; ++q) o[q] += v[q] / (1.f + __expf(-g[q]));
@@ -368,21 +380,24 @@ __global__ void gated_add4_kernel(floatx4* __restrict__ x, const floatx4* __rest
   }
 }
 
-extern "C" int llmlab_gated_add(float* x, const float* y, const float* gate, int gate_cols, const float* bias, int rows,
-                                int width, hipStream_t stream) {
+extern "C" int llmlab_gated_add(float* x, const float* y, int pieces, size_t piece_stride, const float* gate, int gate_cols,
+                                const float* bias, int rows, int width, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && width > 0 && (gate == nullptr || gate_cols == 1 || gate_cols == width),
                  "gated_add: a gate per number or one per row, got %d columns for a width of %d", gate_cols, width);
+  LLMLAB_REQUIRE(pieces >= 1 && pieces <= GATED_ADD_MAX_PIECES, "gated_add: 1 to %d pieces, got %d", GATED_ADD_MAX_PIECES,
+                 pieces);
   const size_t n = (size_t)rows * width;
   if (n == 0) return 0;
-  const bool vec = gate && gate_cols == width && width % 4 == 0 &&
+  const bool vec = gate && gate_cols == width && width % 4 == 0 && piece_stride % 4 == 0 &&
                    (((uintptr_t)x | (uintptr_t)y | (uintptr_t)gate | (uintptr_t)bias) & 15) == 0;
   const size_t work = vec ? n / 4 : n;
   const int blocks = (int)((work + 255) / 256 < 65535 ? (work + 255) / 256 : 65535);
   if (vec)
-    hipLaunchKernelGGL(gated_add4_kernel, dim3(blocks), dim3(256), 0, stream, (floatx4*)x, (const floatx4*)y,
-                       (const floatx4*)gate, (const floatx4*)bias, width / 4, n / 4);
+    hipLaunchKernelGGL(gated_add4_kernel, dim3(blocks), dim3(256), 0, stream, (floatx4*)x, (const floatx4*)y, pieces,
+                       piece_stride / 4, (const floatx4*)gate, (const floatx4*)bias, width / 4, n / 4);
   else
-    hipLaunchKernelGGL(gated_add_kernel, dim3(blocks), dim3(256), 0, stream, x, y, gate, gate_cols, bias, width, n);
+    hipLaunchKernelGGL(gated_add_kernel, dim3(blocks), dim3(256), 0, stream, x, y, pieces, piece_stride, gate, gate_cols,
+                       bias, width, n);
   LLMLAB_LAUNCH_CHECK("gated_add");
   return 0;
 }

@@ -1081,7 +1081,8 @@ class HipOps:
                 lib.llmlab_norm_conv.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                                                  _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
                 lib.llmlab_norm_conv.restype = _c_int
-                lib.llmlab_gated_add.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr]
+                lib.llmlab_gated_add.argtypes = [_c_ptr, _c_ptr, _c_int, _c_size, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
+                                                 _c_ptr]
                 lib.llmlab_gated_add.restype = _c_int
                 lib.llmlab_softcap.argtypes = [_c_ptr, _c_float, _c_size, _c_ptr]
                 lib.llmlab_softcap.restype = _c_int
@@ -1601,13 +1602,24 @@ class HipOps:
                    self._ptr(req_rows), self._ptr(h), self._ptr(out), _dt(h), rows, width, 1 if one_row_each else 0,
                    self._stream(), lib=lib)
 
+    GATED_ADD_MAX_PIECES = 8
+
     def gated_add(self, x, y, gate, bias) -> None:
         """``x += y * sigmoid(gate + bias)``, all float32: ``gate [rows, width]``, or ``[rows, 1]`` for
-        one number a row; ``bias [width]`` or None; ``gate`` None: ``x += y``."""
+        one number a row; ``bias [width]`` or None; ``gate`` None: ``x += y``.  ``y``: a tensor
+        ``[rows, width]``, or the ``PendingSums`` of a product left in up to ``GATED_ADD_MAX_PIECES``
+        pieces, which are summed on the way."""
         lib = self._mixer_lib("stream_ops")
         self._need(x, "residual stream", torch.float32)
-        self._need(y, "sublayer output", torch.float32)
         rows, width = x.shape
+        pieces, piece_stride = 1, 0
+        if isinstance(y, PendingSums):
+            p = y.parts
+            if (p.dtype != torch.float32 or p.dim() != 3 or tuple(p.shape[1:]) != (rows, width) or not p[0].is_contiguous()
+                    or not 1 <= y.splits <= min(p.shape[0], self.GATED_ADD_MAX_PIECES)):
+                raise ValueError(f"gated_add: pieces {tuple(p.shape)} ({y.splits} used) onto {tuple(x.shape)}")
+            pieces, piece_stride, y = y.splits, p.stride(0), p[0]
+        self._need(y, "sublayer output", torch.float32)
         if tuple(y.shape) != (rows, width):
             raise ValueError(f"gated_add: {tuple(y.shape)} onto {tuple(x.shape)}")
         cols = 0
@@ -1620,8 +1632,8 @@ class HipOps:
             self._need(bias, "gate bias", torch.float32)
             if bias.numel() != width or gate is None:
                 raise ValueError("gated_add: a bias per column of a gate")
-        self._call(lib.llmlab_gated_add, self._ptr(x), self._ptr(y), self._ptr(gate), cols, self._ptr(bias), rows, width,
-                   self._stream(), lib=lib)
+        self._call(lib.llmlab_gated_add, self._ptr(x), self._ptr(y), pieces, piece_stride, self._ptr(gate), cols,
+                   self._ptr(bias), rows, width, self._stream(), lib=lib)
 
     def softcap(self, x, cap: float) -> None:
         """``x = cap * tanh(x / cap)`` in place, float32."""

@@ -269,6 +269,14 @@ class GatedConvBlock(Block):
         y = ctx.scratch("block.sublayer_out", (rows, self.hidden_size), torch.float32)
         if part.writes_output:
             part.forward_into(hin, y, ctx, *view)
+        elif hasattr(part, "forward_pending") and hasattr(ops, "GATED_ADD_MAX_PIECES"):
+            # (a product left in pieces is summed by the gated sum itself)
+            pieces = part.forward_pending(hin, y, ctx, *view)
+            if pieces is not None and pieces.splits <= ops.GATED_ADD_MAX_PIECES:
+                y = pieces
+            elif pieces is not None:
+                ops.activation(y, y, "zero")
+                ops.add_pending(y, pieces)
         else:
             ops.activation(y, y, "zero")
             part.forward(hin, y, ctx, *view)

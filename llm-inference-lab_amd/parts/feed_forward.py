@@ -87,6 +87,22 @@ class SwiGLU(FeedForward):
     takes_normed_input = True
     keeps_launches = True
 
+    def forward_pending(self, h, out, ctx):
+        """The result into ``out`` (float32), or, where the down product is left in pieces, the
+        pieces themselves (``PendingSums``; ``out`` is not written): for a caller that does
+        something else with the result than add it to the stream."""
+        rows = h.shape[0]
+        if isinstance(h, NormedInput):
+            h = h.tensor()
+        act = ctx.scratch("swiglu.act", (rows, self.kernel_size), self.dtype)
+        self.ops.linear_swiglu(h, self.w_gate_up, act)
+        splits = self.ops.split_count(rows, self.dtype, self.hidden_size, self.kernel_size)
+        if splits > 1:
+            parts = ctx.scratch("swiglu.pieces", (splits, rows, self.hidden_size), torch.float32)
+            return self.ops.linear_partials(act, self.w_down, parts, splits)
+        self.ops.linear_logits(act, self.w_down, out)
+        return None
+
     def forward(self, h, residual, ctx):
         rows = h.shape[0]
         act = ctx.scratch("swiglu.act", (rows, self.kernel_size), self.dtype)

@@ -475,6 +475,7 @@ class EmuOps:
             state[slot] = joined[-(taps - 1):].to(state.dtype)
 
     NORM_CONV_MAX_TAPS = 8
+    GATED_ADD_MAX_PIECES = 8
 
     def norm_conv(self, x, norm_weight, eps, weight, state, row_req, q_start, req_rows, h, out, one_row_each):
         """The RMS norm of the stream's rows into ``h`` and ``causal_conv`` over them into ``out``."""
@@ -490,6 +491,8 @@ class EmuOps:
         """``x += y * sigmoid(gate + bias)``: ``gate [rows, width]`` or one number a row ``[rows, 1]``
         (None: ``x += y``), all float32."""
         self._count("gated_add")
+        if isinstance(y, PendingSums):
+            y = y.parts[:y.splits].float().sum(0)
         if gate is None:
             x += y
             return

@@ -148,6 +148,15 @@ def test_gated_add(ops, emu, rows, width, cols, bias):
     got = x.to(DEV)
     ops.gated_add(got, *on(DEV, y, gate, b))
     assert (got.cpu() - want).abs().max() <= 1e-5
+    # the same with y left in pieces (the buffer holds more pieces than are used)
+    from llm_inference_lab_amd.parts import PendingSums
+    for pieces in (1, 3, 8):
+        parts = rnd((9, rows, width), torch.float32, 5 + pieces)
+        want = x.clone()
+        emu.gated_add(want, parts[:pieces].sum(0), gate, b)
+        got = x.to(DEV)
+        ops.gated_add(got, PendingSums(parts.to(DEV), pieces), *on(DEV, gate, b))
+        assert (got.cpu() - want).abs().max() <= 2e-5, pieces
 
 
 def test_softcap(ops, emu):
