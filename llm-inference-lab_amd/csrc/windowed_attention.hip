@@ -450,8 +450,8 @@ __global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(MfmaArg
 // Prompts whose heads read the same keys and values (one key/value head, or groups of a multiple
 // of four heads): a block takes 16 consecutive rows and FOUR heads, a wave a head.  The block
 // stages every tile of 32 keys and their values in LDS once (each thread asks for its 16-byte
-// pieces of the next tile before the products of this one and stores them after), and the waves
-// take their fragments from there instead of each from L2.  Key rows lie 16 bytes apart from a
+// pieces two tiles ahead and stores them a tile ahead), and the waves take their fragments from
+// there instead of each from L2.  Key rows lie 16 bytes apart from a
 // multiple of 256 bytes and the values' quad rows 128, so that the lanes of a read spread over the
 // banks.  Everything else (the list of tiles, masks, the running softmax, the transposed
 // products) is the kernel's above; all waves of a block walk the same tiles, so the barriers
@@ -501,9 +501,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
     if (p_hi < 0) continue;
     const KeyTiles kt(p_lo, p_hi, a.window, a.keep_first);
     const int* pages = a.table + (size_t)b * a.max_pages;
-    bf16x8 kreg[KCH], vreg[VCH];
+    // Two sets of staging registers: a tile's pieces are asked for TWO tiles ahead and stored one
+    // tile ahead, so that their way from memory lies behind the products of a whole tile and
+    // more (the longest block's tiles, one after the other, are what a prompt's attention takes).
+    bf16x8 k_a[KCH], v_a[VCH], k_b[KCH], v_b[VCH];
     // the 16-byte pieces of tile t that this thread brings
-    auto fetch = [&](int t) {
+    auto fetch = [&](int t, bf16x8 (&kreg)[KCH], bf16x8 (&vreg)[VCH]) {
       const int j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
       const int end = t < kt.tiles_a ? kt.a_end : kt.end_b;
       size_t kbase[2], vbase[2];
@@ -534,7 +537,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
         vreg[i] = (idx < VCHUNKS && have[u & 1]) ? *(const bf16x8*)(a.v_cache + vbase[u & 1] + (size_t)rem * 8) : zero8;
       }
     };
-    auto stash = [&]() {
+    auto stash = [&](const bf16x8 (&kreg)[KCH], const bf16x8 (&vreg)[VCH]) {
 #pragma unroll
       for (int i = 0; i < KCH; ++i) {
         const int idx = tid + 256 * i;
@@ -554,12 +557,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
         }
       }
     };
-    __syncthreads();                                  // (the request before this one has been read)
-    fetch(0);
-    stash();
-    __syncthreads();
-    for (int t = 0; t < kt.tiles; ++t) {
-      if (t + 1 < kt.tiles) fetch(t + 1);
+    // tile t, which lies in LDS, into the running softmax
+    auto attend = [&](int t) {
       const int j0 = t < kt.tiles_a ? 32 * t : kt.b_start + 32 * (t - kt.tiles_a);
       const int end = t < kt.tiles_a ? kt.a_end : kt.end_b;
       const bool have1 = j0 + 16 < end;
@@ -627,8 +626,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
         for (int i = 0; i < 4; ++i) run.o[eb][i] *= corr;
         run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, run.o[eb], 0, 0, 0);
       }
+    };
+    const int T = kt.tiles;
+    __syncthreads();                                  // (the request before this one has been read)
+    fetch(0, k_a, v_a);
+    stash(k_a, v_a);
+    __syncthreads();
+    if (T > 1) fetch(1, k_a, v_a);
+    for (int t = 0; t < T; t += 2) {
+      // tile t lies in LDS, tile t + 1 is on its way into set a
+      if (t + 2 < T) fetch(t + 2, k_b, v_b);
+      attend(t);
       __syncthreads();                                // (every wave has read the tile)
-      if (t + 1 < kt.tiles) stash();
+      if (t + 1 < T) stash(k_a, v_a);
+      __syncthreads();
+      if (t + 1 >= T) break;
+      // tile t + 1 lies in LDS, tile t + 2 is on its way into set b
+      if (t + 3 < T) fetch(t + 3, k_a, v_a);
+      attend(t + 1);
+      __syncthreads();
+      if (t + 2 < T) stash(k_b, v_b);
       __syncthreads();
     }
   }
