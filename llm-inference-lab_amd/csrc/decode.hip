@@ -89,12 +89,17 @@ struct SkinnyArgs {
   // (no residual, bias in group 0) in out[s][M][ldo], part_stride numbers apart.
   int ksplit;
   size_t part_stride;
-  int act;         // SK_STORE only: 1 = max(z, 0)^2 before the rounding
+  int act;         // SK_STORE: 1 = max(z, 0)^2 before the rounding; SK_SWIGLU: 2 = gelu (tanh form) gate
   int tiles;       // tiles of 16 MB rows
   int col_blocks;  // blocks that a tile of rows takes (sets of columns, times ksplit)
 };
 
 __device__ __forceinline__ float sk_silu(float z) { return z / (1.f + __expf(-z)); }
+// gelu (tanh form), 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), as z * sigmoid(2 t)
+__device__ __forceinline__ float sk_gelu_tanh(float z) {
+  const float t = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return z / (1.f + __expf(-2.f * t));
+}
 
 // Loads of W (and of x where it is not staged) run R steps ahead of the MFMAs in a
 // ring of registers that is refilled slot by slot, so a wave always has R loads
@@ -488,7 +493,7 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
       const int pr = j >> 4, cc = j & 15;
       const float gv = tile[m * cols + pr * 32 + cc], uv = tile[m * cols + pr * 32 + 16 + cc];
       const int o = ((n0 >> 5) + pr) * 16 + cc;
-      if (o < a.n_out) ((bf16_t*)a.out)[(size_t)m * a.ldo + o] = (bf16_t)(sk_silu(gv) * uv);
+      if (o < a.n_out) ((bf16_t*)a.out)[(size_t)m * a.ldo + o] = (bf16_t)((a.act == 2 ? sk_gelu_tanh(gv) : sk_silu(gv)) * uv);
     }
   }
   if constexpr (EPI == SK_QKV) {
@@ -726,8 +731,10 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
                                     hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && M <= SK_MAX_ROWS, "skinny_linear: takes at most %d rows, got %d", SK_MAX_ROWS, M);
   LLMLAB_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny_linear: bad sizes N=%d K=%d (K must be a multiple of 8)", N, K);
-  const int act = epilogue == 6 ? 1 : 0;      // (6 at this interface: STORE through the squared relu)
-  if (act) epilogue = SK_STORE;
+  // (6 at this interface: STORE through the squared relu; 7: the paired product with a gelu gate)
+  const int act = epilogue == 6 ? 1 : epilogue == 7 ? 2 : 0;
+  if (act == 1) epilogue = SK_STORE;
+  if (act == 2) epilogue = SK_SWIGLU;
   LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 5, "skinny_linear: unknown epilogue %d", epilogue);
   LLMLAB_REQUIRE(pend_splits >= 0 && (pend_splits == 0 || (pend != nullptr && (norm || epilogue == SK_RESID))),
                  "skinny_linear: pending sums go with a norm or into the residual");

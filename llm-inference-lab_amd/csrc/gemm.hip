@@ -70,7 +70,8 @@ struct EpiArgs {
   bf16_t* kcache;
   bf16_t* vcache;
   int table_stride, page_size, nq, nkv, d;
-  // STORE only: 1 = the sum goes through max(z, 0)^2 (in float32) before it is rounded
+  // STORE: 1 = the sum goes through max(z, 0)^2 (in float32) before it is rounded;
+  // SWIGLU: 2 = the gate goes through gelu (tanh form) instead of silu
   int act;
   // Grouped products (several matrices of equal shape, one below the other in W; every tile of
   // rows belongs to one of them): g_tile[tile of rows] is the tile's matrix (-1: the tile is
@@ -87,6 +88,21 @@ __device__ __forceinline__ float relu2_f(float z) {
 }
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
+
+// tanh form of gelu: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), as z * sigmoid(2 t)
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  const float t = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return z / (1.f + __expf(-2.f * t));
+}
+__device__ __forceinline__ float gelu_tanh_exact_f(float z) {
+  const float t = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return 0.5f * z * (1.f + tanhf(t));
+}
+// the gate of a paired product: act 2 = gelu (tanh form), else silu
+__device__ __forceinline__ float gate_act_f(float z, int act) { return act == 2 ? gelu_tanh_f(z) : silu_f(z); }
+__device__ __forceinline__ float gate_act_exact_f(float z, int act) {
+  return act == 2 ? gelu_tanh_exact_f(z) : z / (1.f + expf(-z));
+}
 
 // One output element (non-SWIGLU).
 template <typename T, int EPI>
@@ -241,8 +257,8 @@ __device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e,
       bf16x8 v;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        v[q] = (bf16_t)(silu_f(g0[q]) * u0[q]);
-        v[4 + q] = (bf16_t)(silu_f(g1[q]) * u1[q]);
+        v[q] = (bf16_t)(gate_act_f(g0[q], e.act) * u0[q]);
+        v[4 + q] = (bf16_t)(gate_act_f(g1[q], e.act) * u1[q]);
       }
       bf16_t* dst = out + (size_t)m * e.ldo + o0 + oc;
       if (vec && o0 + oc + 8 <= e.n_out) *(bf16x8*)dst = v;
@@ -782,7 +798,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
         const int o = (nb >> 5) * 16 + tx;
         if (o < e.n_out) {
           const float z = acc[i][j];
-          ((float*)e.out)[(size_t)m * e.ldo + o] = z / (1.f + expf(-z)) * acc[i][j + 1];
+          ((float*)e.out)[(size_t)m * e.ldo + o] = gate_act_exact_f(z, e.act) * acc[i][j + 1];
         }
       } else {
         const int n = n0 + tx + 16 * j;
@@ -891,7 +907,7 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
           const int o = (nb >> 5) * 16 + 8 * (x >> 2) + 4 * kk + (x & 3);
           if (o < e.n_out) {
             const float z = acc[j][i][x];
-            ((float*)e.out)[(size_t)m * e.ldo + o] = z / (1.f + expf(-z)) * acc[j][i][x + 8];
+            ((float*)e.out)[(size_t)m * e.ldo + o] = gate_act_exact_f(z, e.act) * acc[j][i][x + 8];
           }
         }
       } else {
@@ -1046,7 +1062,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_f32_rows_kernel(const float* __r
         const int o = (rows_w[j] >> 5) * 16 + (rows_w[j] & 15);
         if (o < e.n_out) {
           const float z = acc[i][j];
-          ((float*)e.out)[(size_t)m * e.ldo + o] = z / (1.f + expf(-z)) * acc[i][j + 2];
+          ((float*)e.out)[(size_t)m * e.ldo + o] = gate_act_exact_f(z, e.act) * acc[i][j + 2];
         }
       }
     } else {
@@ -1452,9 +1468,11 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
                              const void* bias, int bias_dtype, int M, int N, int K, int ldo, int n_out,
                              int num_cus, hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
-  // 6 at this interface: STORE with the squared-relu activation on the way
-  const int act = epilogue == 6 ? 1 : 0;
-  if (act) epilogue = EPI_STORE;
+  // 6 at this interface: STORE with the squared-relu activation on the way; 7: the paired
+  // product whose gate goes through gelu (tanh form)
+  const int act = epilogue == 6 ? 1 : epilogue == 7 ? 2 : 0;
+  if (act == 1) epilogue = EPI_STORE;
+  if (act == 2) epilogue = EPI_SWIGLU;
   LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 3, "linear: unknown epilogue %d", epilogue);
   if (epilogue == EPI_SWIGLU) {
     LLMLAB_REQUIRE(N % 32 == 0 && n_out > 0 && 2 * ((n_out + 15) / 16 * 16) == N,

@@ -240,13 +240,14 @@ extern "C" int llmlab_gla_scan(const float* proj, int ld, int off_q, int off_k, 
 
 // ---------------------------------------------------------------------- output
 // Block (row, head): o = sum over slices of parts; y = o / sqrt(mean(o^2) + eps) * w[e]
-// (the weight has one entry per value channel, the same for every head); out = T(y *
-// silu(gate)), silu(g) = g / (1 + exp(-g)); gate [rows, ld] float32 at column off_g.
+// (the weight has one entry per value channel, the same for every head; w_per_head: one per
+// head and channel, w[h * E + e]); out = T(y * silu(gate)), silu(g) = g / (1 + exp(-g))
+// (gate_kind 1: y * sigmoid(gate)); gate [rows, ld] float32 at column off_g.
 template <typename T>
 __global__ __launch_bounds__(1024) void gla_output_kernel(const float* __restrict__ parts, int slices, int n_heads, int E,
                                                           const float* __restrict__ w, float eps,
                                                           const float* __restrict__ proj, int ld, int off_g,
-                                                          T* __restrict__ out) {
+                                                          T* __restrict__ out, int w_per_head, int gate_kind) {
   __shared__ float red[17];
   const int r = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
   float o = 0.f;
@@ -257,24 +258,161 @@ __global__ __launch_bounds__(1024) void gla_output_kernel(const float* __restric
   const float ms = block_sum(o * o, red) / (float)E;
   if (e < E) {
     const float g = proj[(size_t)r * ld + off_g + h * E + e];
-    const float y = o * (1.0f / sqrtf(ms + eps)) * w[e];
-    out[((size_t)r * n_heads + h) * E + e] = from_float<T>(y * (g / (1.0f + expf(-g))));
+    const float y = o * (1.0f / sqrtf(ms + eps)) * w[w_per_head ? h * E + e : e];
+    const float sg = 1.0f / (1.0f + expf(-g));
+    out[((size_t)r * n_heads + h) * E + e] = from_float<T>(y * (gate_kind == 1 ? sg : g * sg));
   }
 }
 
+// slices > 0: that many pieces per output (0: as the gated scan leaves them, one per SLICE key channels)
 extern "C" int llmlab_gla_output(const float* parts, int rows, int n_heads, int D, int E, const float* w, float eps,
-                                 const float* proj, int ld, int off_g, void* out, int dtype, hipStream_t stream) {
+                                 const float* proj, int ld, int off_g, void* out, int dtype, int slices_given,
+                                 int w_per_head, int gate_kind, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && n_heads > 0 && n_heads <= 65535 && E > 0 && E <= 1024,
                  "gla_output: bad sizes rows=%d heads=%d E=%d", rows, n_heads, E);
+  LLMLAB_REQUIRE(gate_kind == 0 || gate_kind == 1, "gla_output: unknown gate %d", gate_kind);
   if (rows == 0) return 0;
-  const int slices = (D + SLICE - 1) / SLICE;
+  const int slices = slices_given > 0 ? slices_given : (D + SLICE - 1) / SLICE;
   dim3 grid(rows, n_heads), block((E + 63) / 64 * 64);
   if (dtype == DT_BF16)
     hipLaunchKernelGGL(gla_output_kernel<bf16_t>, grid, block, 0, stream, parts, slices, n_heads, E, w, eps, proj, ld,
-                       off_g, (bf16_t*)out);
+                       off_g, (bf16_t*)out, w_per_head, gate_kind);
   else
     hipLaunchKernelGGL(gla_output_kernel<float>, grid, block, 0, stream, parts, slices, n_heads, E, w, eps, proj, ld,
-                       off_g, (float*)out);
+                       off_g, (float*)out, w_per_head, gate_kind);
   LLMLAB_LAUNCH_CHECK("gla_output");
+  return 0;
+}
+
+
+// ================================================================== generalised delta rule
+// A matrix-valued state per head whose transition is a decay per key channel less a rank-one
+// removal along the unit key, before the new key/value pair is written:
+//   u_t = k_t / sqrt(|k_t|^2 + key_eps)
+//   S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T        (both terms read S_(t-1))
+//   o_t = S_t^T r_t
+// with w_t (decay) and a_t (removal rate) in (0, 1) per head and key channel.  State [D, E]
+// per head, float32, one slot per request; everything here is float32.
+//
+// delta_gates: w = exp(-decay_scale * sigmoid(w0 + W2 tanh(low))) from the low-rank projection
+// `low` (rank numbers a row), a = sigmoid(a_in + a_bias).
+__global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restrict__ proj, int ld, int off_low, int rank,
+                                                          int off_a, const float* __restrict__ w2,
+                                                          const float* __restrict__ w0, const float* __restrict__ a_bias,
+                                                          float decay_scale, float* __restrict__ decay,
+                                                          float* __restrict__ rate, int channels) {
+  extern __shared__ float s_low[];       // tanh of the row's low-rank numbers
+  const int r = blockIdx.x;
+  const float* t = proj + (size_t)r * ld;
+  for (int j = threadIdx.x; j < rank; j += blockDim.x) s_low[j] = tanhf(t[off_low + j]);
+  __syncthreads();
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    float z = w0 ? w0[c] : 0.f;
+    const float* w = w2 + (size_t)c * rank;
+    for (int j = 0; j < rank; ++j) z = fmaf(w[j], s_low[j], z);
+    decay[(size_t)r * channels + c] = expf(-decay_scale / (1.0f + expf(-z)));
+    const float za = t[off_a + c] + (a_bias ? a_bias[c] : 0.f);
+    rate[(size_t)r * channels + c] = 1.0f / (1.0f + expf(-za));
+  }
+}
+
+extern "C" int llmlab_delta_gates(const float* proj, int ld, int rows, int off_low, int rank, int off_a, const float* w2,
+                                  const float* w0, const float* a_bias, float decay_scale, float* decay, float* rate,
+                                  int channels, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && rank > 0 && rank <= 8192 && channels > 0 && off_low >= 0 && off_a >= 0 &&
+                 ld >= off_low + rank && ld >= off_a + channels,
+                 "delta_gates: bad sizes rows=%d rank=%d channels=%d ld=%d", rows, rank, channels, ld);
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(delta_gates_kernel, dim3(rows), dim3(256), rank * sizeof(float), stream, proj, ld, off_low, rank,
+                     off_a, w2, w0, a_bias, decay_scale, decay, rate, channels);
+  LLMLAB_LAUNCH_CHECK("delta_gates");
+  return 0;
+}
+
+// delta_scan: thread e of block (request, head) keeps column e of the head's state (DK >= D
+// numbers) in registers and walks the request's rows of the step in order; the row's key,
+// receptance, decay and rate are the same for every thread of the block (uniform loads), its
+// value is one number a thread.  No thread talks to another, so a token costs no barrier.
+// Rows [row_begin, row_end) of the request: the state comes from `s_in` and goes to `s_out`
+// (both [D, E] of this head; s_in null: zero).
+template <int DK>
+__device__ __forceinline__ void delta_walk(const float* __restrict__ proj, int ld, int off_r, int off_k, int off_v,
+                                           const float* __restrict__ decay, const float* __restrict__ rate, int n_heads,
+                                           int h, int D, int E, float key_eps, int row_begin, int row_end,
+                                           const float* __restrict__ s_in, float* __restrict__ s_out,
+                                           float* __restrict__ out, int e) {
+  float S[DK];
+#pragma unroll
+  for (int d = 0; d < DK; ++d) S[d] = (s_in && d < D && e < E) ? s_in[(size_t)d * E + e] : 0.f;
+  const int ec = e < E ? e : E - 1;
+  for (int t = row_begin; t < row_end; ++t) {
+    const float* row = proj + (size_t)t * ld;
+    const float* kk = row + off_k + h * D;
+    const float* rr = row + off_r + h * D;
+    const float* ww = decay + ((size_t)t * n_heads + h) * D;
+    const float* aa = rate + ((size_t)t * n_heads + h) * D;
+    const float v = row[off_v + h * E + ec];
+    float k2 = 0.f;
+#pragma unroll
+    for (int d = 0; d < DK; ++d)
+      if (d < D) k2 = fmaf(kk[d], kk[d], k2);
+    const float inv = 1.0f / sqrtf(k2 + key_eps);
+    float dot = 0.f;
+#pragma unroll
+    for (int d = 0; d < DK; ++d)
+      if (d < D) dot = fmaf(kk[d] * inv, S[d], dot);
+    float o = 0.f;
+#pragma unroll
+    for (int d = 0; d < DK; ++d)
+      if (d < D) {
+        const float k = kk[d];
+        S[d] = fmaf(ww[d], S[d], fmaf(-(aa[d] * (k * inv)), dot, k * v));
+        o = fmaf(S[d], rr[d], o);
+      }
+    if (e < E) out[((size_t)t * n_heads + h) * E + e] = o;
+  }
+  if (e < E) {
+#pragma unroll
+    for (int d = 0; d < DK; ++d)
+      if (d < D) s_out[(size_t)d * E + e] = S[d];
+  }
+}
+
+template <int DK>
+__global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ proj, int ld, int off_r, int off_k,
+                                                         int off_v, const float* __restrict__ decay,
+                                                         const float* __restrict__ rate, int n_heads, int D, int E,
+                                                         float key_eps, float* __restrict__ state,
+                                                         const int* __restrict__ q_start, const int* __restrict__ req_rows,
+                                                         float* __restrict__ out) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int e = blockIdx.z * blockDim.x + threadIdx.x;
+  float* st = state + ((size_t)req_rows[b] * n_heads + h) * D * E;
+  delta_walk<DK>(proj, ld, off_r, off_k, off_v, decay, rate, n_heads, h, D, E, key_eps, q_start[b], q_start[b + 1], st, st,
+                 out, e);
+}
+
+extern "C" int llmlab_delta_scan(const float* proj, int ld, int off_r, int off_k, int off_v, const float* decay,
+                                 const float* rate, int n_heads, int D, int E, float key_eps, float* state,
+                                 const int* q_start, const int* req_rows, int n_reqs, float* out, int rows,
+                                 hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && n_reqs >= 0 && n_heads > 0 && n_heads <= 65535 && D > 0 && D <= 256 && E > 0 && E <= 16384,
+                 "delta_scan: bad sizes rows=%d requests=%d heads=%d D=%d E=%d (keys up to 256 wide)", rows, n_reqs,
+                 n_heads, D, E);
+  LLMLAB_REQUIRE(off_r >= 0 && off_k >= 0 && off_v >= 0 && ld >= off_r + n_heads * D && ld >= off_k + n_heads * D &&
+                 ld >= off_v + n_heads * E, "delta_scan: rows of %d numbers do not hold the projections", ld);
+  if (rows == 0 || n_reqs == 0) return 0;
+  const int threads = E <= 64 ? 64 : (E <= 128 ? 128 : 256);
+  dim3 grid(n_reqs, n_heads, (E + threads - 1) / threads), block(threads);
+#define LLMLAB_DELTA(DKV)                                                                                             \
+  hipLaunchKernelGGL(delta_scan_kernel<DKV>, grid, block, 0, stream, proj, ld, off_r, off_k, off_v, decay, rate, n_heads, \
+                     D, E, key_eps, state, q_start, req_rows, out)
+  if (D <= 16) LLMLAB_DELTA(16);
+  else if (D <= 32) LLMLAB_DELTA(32);
+  else if (D <= 64) LLMLAB_DELTA(64);
+  else if (D <= 128) LLMLAB_DELTA(128);
+  else LLMLAB_DELTA(256);
+#undef LLMLAB_DELTA
+  LLMLAB_LAUNCH_CHECK("delta_scan");
   return 0;
 }

@@ -4,6 +4,8 @@
 //   norm_conv       the RMS norm of the stream's rows and that convolution over them in one launch
 //   gated_add       x += y * sigmoid(gate + bias)
 //   softcap         x = cap * tanh(x / cap)
+//   rmsnorm_add     x += y / sqrt(mean(y^2) + eps) * w   (a norm on a sublayer's result, before the sum)
+//   scaled_sum      out = a * y1 + b * y2
 // What a request's earlier steps left (its last token, the last inputs of a convolution) lives in
 // per-request slots; a step's rows of one request are adjacent.
 #include "common.h"
@@ -399,6 +401,69 @@ extern "C" int llmlab_gated_add(float* x, const float* y, int pieces, size_t pie
     hipLaunchKernelGGL(gated_add_kernel, dim3(blocks), dim3(256), 0, stream, x, y, pieces, piece_stride, gate, gate_cols,
                        bias, width, n);
   LLMLAB_LAUNCH_CHECK("gated_add");
+  return 0;
+}
+
+// ------------------------------------------------------------------ norm of a sublayer's result into the stream
+// One block a row: x[r, c] += v[c] / sqrt(mean(v^2) + eps) * w[c] with v = y[r] (or the sum of its
+// pieces, in the pieces' order).  All float32.  A thread keeps up to NORM_ADD_KEEP of the row's numbers
+// in registers between the two passes; wider rows are read again.
+constexpr int NORM_ADD_KEEP = 8;
+__global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y, int pieces,
+                                                          size_t piece_stride, const float* __restrict__ w, float eps,
+                                                          int width) {
+  __shared__ float red[17];
+  const size_t row = (size_t)blockIdx.x * width;
+  float keep[NORM_ADD_KEEP];
+  float ss = 0.f;
+  auto value = [&](int c) {
+    float v = y[row + c];
+    for (int s = 1; s < pieces; ++s) v += y[s * piece_stride + row + c];
+    return v;
+  };
+#pragma unroll
+  for (int n = 0; n < NORM_ADD_KEEP; ++n) {
+    const int c = threadIdx.x + 256 * n;
+    keep[n] = c < width ? value(c) : 0.f;
+    ss = fmaf(keep[n], keep[n], ss);
+  }
+  for (int c = threadIdx.x + 256 * NORM_ADD_KEEP; c < width; c += 256) {
+    const float v = value(c);
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)width + eps);
+#pragma unroll
+  for (int n = 0; n < NORM_ADD_KEEP; ++n) {
+    const int c = threadIdx.x + 256 * n;
+    if (c < width) x[row + c] += keep[n] * inv * w[c];
+  }
+  for (int c = threadIdx.x + 256 * NORM_ADD_KEEP; c < width; c += 256) x[row + c] += value(c) * inv * w[c];
+}
+
+extern "C" int llmlab_rmsnorm_add(float* x, const float* y, int pieces, size_t piece_stride, const float* w, float eps,
+                                  int rows, int width, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && width > 0 && pieces >= 1 && x && y && w, "rmsnorm_add: bad arguments rows=%d width=%d pieces=%d",
+                 rows, width, pieces);
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(rows), dim3(256), 0, stream, x, y, pieces, piece_stride, w, eps, width);
+  LLMLAB_LAUNCH_CHECK("rmsnorm_add");
+  return 0;
+}
+
+// ------------------------------------------------------------------ two results side by side
+__global__ void scaled_sum_kernel(float* __restrict__ out, const float* __restrict__ y1, float a,
+                                  const float* __restrict__ y2, float b, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    out[i] = a * y1[i] + b * y2[i];
+}
+
+extern "C" int llmlab_scaled_sum(float* out, const float* y1, float a, const float* y2, float b, size_t n,
+                                 hipStream_t stream) {
+  LLMLAB_REQUIRE(out && y1 && y2, "scaled_sum: null operand");
+  if (n == 0) return 0;
+  const int blocks = (int)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  hipLaunchKernelGGL(scaled_sum_kernel, dim3(blocks), dim3(256), 0, stream, out, y1, a, y2, b, n);
+  LLMLAB_LAUNCH_CHECK("scaled_sum");
   return 0;
 }
 

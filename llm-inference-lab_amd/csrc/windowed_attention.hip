@@ -88,6 +88,106 @@ extern "C" int llmlab_project_norm_write(const float* proj, int ld, int rows, in
   return 0;
 }
 
+// The same for layers that turn their queries and keys by position and may mix their values
+// with an earlier layer's.  proj[r, :] = q | k | v | gates (float32 sums); `bias` (float32, the
+// same order, or null) is added first.  Rotation: of every query and key head the first rot_dims
+// channels turn, channel 2i together with channel 2i + 1, by the angle positions[r] * freq[i]
+// (float32), (u, v) -> (u cos - v sin, v cos + u sin), sine and cosine times `magnitude`; the
+// other channels pass.  Values: mix 1 also leaves them, unrounded, in v_first[r]; mix 2 takes
+// v <- (1 - lambda) v + lambda v_first[r] before they are stored.  The n_gate numbers behind the
+// values go to gate_out [rows, n_gate] as they are.
+constexpr int ROTATE_MAX_PAIRS = 256;
+template <typename T>
+__global__ __launch_bounds__(256) void project_rotate_write_kernel(
+    const float* __restrict__ proj, int ld, int n_heads, int n_kv, int D, int E, const float* __restrict__ bias,
+    const float* __restrict__ freq, int rot_dims, float magnitude, int mix, float lambda, float* __restrict__ v_first,
+    int n_gate, float* __restrict__ gate_out, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    int page_size, const int* __restrict__ positions, const int* __restrict__ row_req, const int* __restrict__ table,
+    int max_pages) {
+  __shared__ float s_cos[ROTATE_MAX_PAIRS], s_sin[ROTATE_MAX_PAIRS];
+  const int r = blockIdx.x;
+  const float* src = proj + (size_t)r * ld;
+  const int pos = positions[r];
+  const int half = rot_dims >> 1;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float angle = (float)pos * freq[i];
+    float sn, cs;
+    sincosf(angle, &sn, &cs);
+    s_cos[i] = cs * magnitude;
+    s_sin[i] = sn * magnitude;
+  }
+  __syncthreads();
+  const int q_size = n_heads * D, k_size = n_kv * D, v_size = n_kv * E;
+  const int page = table[(size_t)row_req[r] * max_pages + pos / page_size];
+  const int slot = pos % page_size;
+  // queries and keys, a pair of channels a thread (D even where anything turns)
+  const int pairs_per_head = (D + 1) >> 1;
+  for (int p = threadIdx.x; p < (n_heads + n_kv) * pairs_per_head; p += blockDim.x) {
+    const int hd = p / pairs_per_head, i = p - hd * pairs_per_head;
+    const int c0 = hd * D + 2 * i;
+    const bool two = 2 * i + 1 < D;
+    float u = src[c0] + (bias ? bias[c0] : 0.f);
+    float v = two ? src[c0 + 1] + (bias ? bias[c0 + 1] : 0.f) : 0.f;
+    if (i < half) {
+      const float cs = s_cos[i], sn = s_sin[i];
+      const float u2 = u * cs - v * sn;
+      v = v * cs + u * sn;
+      u = u2;
+    }
+    if (hd < n_heads) {
+      q_out[(size_t)r * q_size + c0] = from_float<T>(u);
+      if (two) q_out[(size_t)r * q_size + c0 + 1] = from_float<T>(v);
+    } else {
+      const int g = hd - n_heads;
+      T* dst = k_cache + (((size_t)page * n_kv + g) * page_size + slot) * D + 2 * i;
+      dst[0] = from_float<T>(u);
+      if (two) dst[1] = from_float<T>(v);
+    }
+  }
+  for (int c = threadIdx.x; c < v_size; c += blockDim.x) {
+    const int g = c / E, e = c - g * E;
+    const int at = q_size + k_size + c;
+    float v = src[at] + (bias ? bias[at] : 0.f);
+    if (mix == 1) v_first[(size_t)r * v_size + c] = v;
+    if (mix == 2) v = (1.f - lambda) * v + lambda * v_first[(size_t)r * v_size + c];
+    v_cache[((size_t)page * n_kv + g) * page_size * E + value_index(slot, e, E)] = from_float<T>(v);
+  }
+  for (int c = threadIdx.x; c < n_gate; c += blockDim.x) {
+    const int at = q_size + k_size + v_size + c;
+    gate_out[(size_t)r * n_gate + c] = src[at] + (bias ? bias[at] : 0.f);
+  }
+}
+
+extern "C" int llmlab_project_rotate_write(const float* proj, int ld, int rows, int n_heads, int n_kv, int D, int E,
+                                           const float* bias, const float* freq, int rot_dims, float magnitude,
+                                           int mix, float lambda, float* v_first, int n_gate, float* gate_out,
+                                           void* q_out, void* k_cache, void* v_cache, int dtype, int page_size,
+                                           const int* positions, const int* row_req, const int* table, int max_pages,
+                                           hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && n_heads > 0 && n_kv > 0 && D > 0 && E > 0 && page_size > 0 && page_size % 4 == 0,
+                 "project_rotate_write: bad sizes rows=%d heads=%d kv=%d D=%d E=%d page=%d", rows, n_heads, n_kv, D, E,
+                 page_size);
+  LLMLAB_REQUIRE(ld >= (n_heads + n_kv) * D + n_kv * E + n_gate && n_gate >= 0,
+                 "project_rotate_write: rows of %d numbers do not hold the projections", ld);
+  LLMLAB_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= D && rot_dims <= 2 * ROTATE_MAX_PAIRS &&
+                 (rot_dims == 0 || freq), "project_rotate_write: %d of %d channels cannot turn in pairs", rot_dims, D);
+  LLMLAB_REQUIRE(mix >= 0 && mix <= 2 && (mix == 0 || v_first), "project_rotate_write: mixed values need the first layer's");
+  LLMLAB_REQUIRE(n_gate == 0 || gate_out, "project_rotate_write: gates need a place");
+  LLMLAB_REQUIRE(q_out && k_cache && v_cache && positions && row_req && table,
+                 "project_rotate_write: queries, pages, positions and the block table are needed");
+  if (rows == 0) return 0;
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(project_rotate_write_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, proj, ld, n_heads, n_kv, D, E,
+                       bias, freq, rot_dims, magnitude, mix, lambda, v_first, n_gate, gate_out, (bf16_t*)q_out,
+                       (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, positions, row_req, table, max_pages);
+  else
+    hipLaunchKernelGGL(project_rotate_write_kernel<float>, dim3(rows), dim3(256), 0, stream, proj, ld, n_heads, n_kv, D, E,
+                       bias, freq, rot_dims, magnitude, mix, lambda, v_first, n_gate, gate_out, (float*)q_out,
+                       (float*)k_cache, (float*)v_cache, page_size, positions, row_req, table, max_pages);
+  LLMLAB_LAUNCH_CHECK("project_rotate_write");
+  return 0;
+}
+
 static int g_force_plain = 0;      // tests and measurements: no matrix-core kernel
 extern "C" void llmlab_debug_windowed_attention_plain(int on) { g_force_plain = on; }
 static int g_private_tiles = 0;    // tests and measurements: prompts by the kernel whose waves fetch their own tiles
@@ -98,6 +198,12 @@ extern "C" void llmlab_debug_windowed_attention_private_tiles(int on) { g_privat
 // kept prefix j < min(keep_first, i + 1); window <= 0: every j <= i.  Scores, the running maximum, the denominator
 // and the weighted sum of values are float32.  With a sink the running maximum starts at
 // sink[h] and the denominator at 1 = exp(sink - sink), and nothing is added to the weighted sum.
+// mode 1 (MODE_SIGMOID): no softmax; the weight of a visible key is sigmoid(score + sink[h])
+// (sink: then a bias per head added to every score, null for none), and the weights are not
+// normalised.  The kernels then keep the running maximum at 0 and the denominator at 1, so the
+// merge of shares and the final division stay as they are.
+constexpr int MODE_SOFTMAX = 0, MODE_SIGMOID = 1;
+__device__ __forceinline__ float sigmoid_weight(float s) { return 1.0f / (1.0f + __expf(-s)); }      // (-inf -> 0)
 //
 // Both kernels walk the keys in two runs, each from an aligned start, and mask key by key:
 // the kept prefix [0, min(keep_first, B)) and [B, i], where B is the window's first key
@@ -160,7 +266,8 @@ __global__ __launch_bounds__(64) void sink_window_attention_kernel(
     const T* __restrict__ q, int n_heads, int n_kv, int D, int E, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ table, int max_pages, int page_size,
     const int* __restrict__ positions, const int* __restrict__ row_req, int window, int keep_first,
-    const float* __restrict__ sink, float scale, T* __restrict__ out, const int* __restrict__ q_start, int long_from) {
+    const float* __restrict__ sink, float scale, T* __restrict__ out, const int* __restrict__ q_start, int long_from,
+    int mode) {
   if (long_from > 0) {      // (rows of requests that bring many rows are the other kernel's)
     const int b = row_req[blockIdx.x];
     if (q_start[b + 1] - q_start[b] >= long_from) return;
@@ -178,8 +285,10 @@ __global__ __launch_bounds__(64) void sink_window_attention_kernel(
   const int lo = window > 0 ? (i - window + 1 > 0 ? i - window + 1 : 0) : 0;
   const int b_start = lo & ~3;
   const int a_end = keep_first < b_start ? keep_first : b_start;
-  float m = sink ? sink[h] : NEG_INF;
-  float l = sink ? 1.f : 0.f;
+  const bool sig = mode == MODE_SIGMOID;
+  const float bias = (sig && sink) ? sink[h] : 0.f;
+  float m = sig ? 0.f : (sink ? sink[h] : NEG_INF);
+  float l = (sig || sink) ? 1.f : 0.f;
   float acc[MAX_E_PER_LANE];
 #pragma unroll
   for (int c = 0; c < MAX_E_PER_LANE; ++c) acc[c] = 0.f;
@@ -196,11 +305,17 @@ __global__ __launch_bounds__(64) void sink_window_attention_kernel(
         if (valid) s = dot_row<T>(qs, k_cache + (head + (j % page_size)) * D, D);
         vquad[lane] = head * E + value_index(j % page_size, 0, E);       // (lanes 4 n are read below)
       }
-      const float m_new = fmaxf(m, wave_max(s));
-      const float p = valid ? __expf(s - m_new) : 0.f;
-      const float corr = (m == NEG_INF) ? 0.f : __expf(m - m_new);
-      l = l * corr + wave_sum(p);
-      m = m_new;
+      float p, corr;
+      if (sig) {
+        p = valid ? sigmoid_weight(s + bias) : 0.f;
+        corr = 1.f;
+      } else {
+        const float m_new = fmaxf(m, wave_max(s));
+        p = valid ? __expf(s - m_new) : 0.f;
+        corr = (m == NEG_INF) ? 0.f : __expf(m - m_new);
+        l = l * corr + wave_sum(p);
+        m = m_new;
+      }
       ps[lane] = p;
       __syncthreads();
       const int quads = ((end - base < 64 ? end - base : 64) + 3) >> 2;
@@ -306,7 +421,8 @@ template <int DC, int EB>
 __device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, int t_end, const bf16x8 (&qf)[DC], bool seen,
                                              int pos, const int* __restrict__ pages, int page_size, int n_kv, int g,
                                              const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
-                                             int window, int keep_first, float scale, Running<EB>& run) {
+                                             int window, int keep_first, float scale, Running<EB>& run,
+                                             int mode, float bias) {
   constexpr int E = 16 * EB;
   const int lane = threadIdx.x & 63, c = lane & 15, g4 = lane >> 4;
   if (t_begin >= t_end) return;
@@ -356,13 +472,22 @@ __device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, in
           tmax = fmaxf(tmax, s[u][i]);
         }
     }
+    bf16x8 pf;
+    if (mode == MODE_SIGMOID) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pf[4 * u + i] = (bf16_t)sigmoid_weight(s[u][i] + bias);      // (masked: -inf -> 0)
+#pragma unroll
+      for (int eb = 0; eb < EB; ++eb)
+        run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[eb], pf, run.o[eb], 0, 0, 0);
+    } else {
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
     const float m_new = fmaxf(run.m, tmax);
     const float m_use = m_new == NEG_INF ? 0.f : m_new;
     const float corr = run.m == NEG_INF ? 0.f : __expf(run.m - m_use);
     float sum = 0.f;
-    bf16x8 pf;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -381,6 +506,7 @@ __device__ __forceinline__ void attend_tiles(const KeyTiles& kt, int t_begin, in
       for (int i = 0; i < 4; ++i) run.o[eb][i] *= corr;
       run.o[eb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[eb], pf, run.o[eb], 0, 0, 0);
     }
+    }
     cur = nxt;
   }
 }
@@ -391,6 +517,7 @@ struct MfmaArgs {
   const int* positions; const int* row_req; int window, keep_first; const float* sink; float scale;
   bf16_t* out; const int* q_start; int long_from;
   int splits; float* part_o; float* part_ml;      // (decoding) [rows, heads, splits, E] and [rows, heads, splits, 2]
+  int mode;                                       // MODE_SOFTMAX, or MODE_SIGMOID (sink: the bias of the scores)
 };
 
 // Prompts: a wave takes 16 consecutive rows and one head, a block four such tiles.  Rows of
@@ -415,8 +542,10 @@ __global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(MfmaArg
       for (int i = 0; i < 8; ++i) qf[dc][i] = (bf16_t)0.f;
   }
   Running<EB> run;
-  run.m = a.sink ? a.sink[h] : NEG_INF;
-  run.l = a.sink ? 1.f : 0.f;
+  const bool sig = a.mode == MODE_SIGMOID;
+  const float bias = (sig && a.sink) ? a.sink[h] : 0.f;
+  run.m = sig ? 0.f : (a.sink ? a.sink[h] : NEG_INF);
+  run.l = (sig || a.sink) ? 1.f : 0.f;
 #pragma unroll
   for (int eb = 0; eb < EB; ++eb) run.o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int b_first = __builtin_amdgcn_readfirstlane(a.row_req[r0]);
@@ -433,7 +562,7 @@ __global__ __launch_bounds__(256) void sink_window_attention_mfma_kernel(MfmaArg
     if (p_hi < 0) continue;
     const KeyTiles kt(p_lo, p_hi, a.window, a.keep_first);
     attend_tiles<DC, EB>(kt, 0, kt.tiles, qf, mine, pos, a.table + (size_t)b * a.max_pages, a.page_size, a.n_kv, g,
-                         a.k_cache, a.v_cache, a.window, a.keep_first, a.scale, run);
+                         a.k_cache, a.v_cache, a.window, a.keep_first, a.scale, run, a.mode, bias);
   }
   if (!row_ok) return;
   if (a.long_from > 0 && a.q_start[req + 1] - a.q_start[req] < a.long_from) return;
@@ -483,8 +612,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
   for (int dc = 0; dc < DC; ++dc)
     qf[dc] = row_ok ? *(const bf16x8*)(a.q + ((size_t)r * a.n_heads + h) * D + 32 * dc + 8 * g4) : zero8;
   Running<EB> run;
-  run.m = a.sink ? a.sink[h] : NEG_INF;
-  run.l = a.sink ? 1.f : 0.f;
+  const bool sig = a.mode == MODE_SIGMOID;
+  const float bias = (sig && a.sink) ? a.sink[h] : 0.f;
+  run.m = sig ? 0.f : (a.sink ? a.sink[h] : NEG_INF);
+  run.l = (sig || a.sink) ? 1.f : 0.f;
 #pragma unroll
   for (int eb = 0; eb < EB; ++eb) run.o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
   const int b_first = __builtin_amdgcn_readfirstlane(a.row_req[r0]);
@@ -594,13 +725,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
             tmax = fmaxf(tmax, s[u][i]);
           }
       }
+      float corr = 1.f;
+      bf16x8 pf;
+      if (a.mode == MODE_SIGMOID) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pf[4 * u + i] = (bf16_t)sigmoid_weight(s[u][i] + bias);      // (masked: -inf -> 0)
+      } else {
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
       const float m_new = fmaxf(run.m, tmax);
       const float m_use = m_new == NEG_INF ? 0.f : m_new;
-      const float corr = run.m == NEG_INF ? 0.f : __expf(run.m - m_use);
+      corr = run.m == NEG_INF ? 0.f : __expf(run.m - m_use);
       float sum = 0.f;
-      bf16x8 pf;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -613,6 +751,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void s
       sum += __shfl_xor(sum, 32, WAVE);
       run.l = run.l * corr + sum;
       run.m = m_new;
+      }
 #pragma unroll
       for (int eb = 0; eb < EB; ++eb) {
         bf16x8 vf;
@@ -689,15 +828,17 @@ __global__ __launch_bounds__(64) void sink_window_attention_grouped_kernel(MfmaA
   }
   const int z = blockIdx.z;
   Running<EB> run;
-  run.m = (a.sink && head_ok && z == 0) ? a.sink[h] : NEG_INF;
-  run.l = (a.sink && head_ok && z == 0) ? 1.f : 0.f;
+  const bool sig = a.mode == MODE_SIGMOID;
+  const float bias = (sig && a.sink && head_ok) ? a.sink[h] : 0.f;
+  run.m = sig ? 0.f : ((a.sink && head_ok && z == 0) ? a.sink[h] : NEG_INF);
+  run.l = sig ? (z == 0 ? 1.f : 0.f) : ((a.sink && head_ok && z == 0) ? 1.f : 0.f);
 #pragma unroll
   for (int eb = 0; eb < EB; ++eb) run.o[eb] = floatx4{0.f, 0.f, 0.f, 0.f};
   const KeyTiles kt(pos, pos, a.window, a.keep_first);
   const int per = (kt.tiles + a.splits - 1) / a.splits;
   const int t_begin = z * per, t_end = (z + 1) * per < kt.tiles ? (z + 1) * per : kt.tiles;
   attend_tiles<DC, EB>(kt, t_begin, t_end, qf, head_ok, pos, a.table + (size_t)b * a.max_pages, a.page_size, a.n_kv, g,
-                       a.k_cache, a.v_cache, a.window, a.keep_first, a.scale, run);
+                       a.k_cache, a.v_cache, a.window, a.keep_first, a.scale, run, a.mode, bias);
   if (!head_ok) return;
   if (a.splits == 1) {
     const float inv = 1.0f / run.l;
@@ -826,8 +967,9 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
                                             int page_size, const int* positions, const int* row_req, int window,
                                             int keep_first, const float* sink, float scale, void* out,
                                             const int* q_start, int long_from, int launches, int max_keys,
-                                            float* workspace, size_t workspace_floats, int num_cus,
+                                            float* workspace, size_t workspace_floats, int num_cus, int mode,
                                             hipStream_t stream) {
+  LLMLAB_REQUIRE(mode == MODE_SOFTMAX || mode == MODE_SIGMOID, "sink_window_attention: unknown weighting %d", mode);
   LLMLAB_REQUIRE(rows >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0 && D > 0 && E > 0,
                  "sink_window_attention: bad sizes rows=%d heads=%d kv=%d D=%d E=%d", rows, n_heads, n_kv, D, E);
   LLMLAB_REQUIRE(E <= 64 * MAX_E_PER_LANE, "sink_window_attention: values up to %d wide, got %d", 64 * MAX_E_PER_LANE, E);
@@ -843,7 +985,7 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
   if (long_from > 0) {
     MfmaArgs a{(const bf16_t*)q, rows, n_heads, n_kv, (const bf16_t*)k_cache, (const bf16_t*)v_cache, table, max_pages,
                page_size, positions, row_req, window, keep_first, sink, scale, (bf16_t*)out, q_start, long_from, 1,
-               nullptr, nullptr};
+               nullptr, nullptr, mode};
     if (launches & 2) {
       // heads that read the same keys and values share the tiles a block stages in LDS
       const int group = n_heads / n_kv;
@@ -884,11 +1026,11 @@ extern "C" int llmlab_sink_window_attention(const void* q, int dtype, int rows, 
   if (dtype == DT_BF16)
     hipLaunchKernelGGL(sink_window_attention_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)q, n_heads, n_kv, D,
                        E, (const bf16_t*)k_cache, (const bf16_t*)v_cache, table, max_pages, page_size, positions,
-                       row_req, window, keep_first, sink, scale, (bf16_t*)out, q_start, long_from);
+                       row_req, window, keep_first, sink, scale, (bf16_t*)out, q_start, long_from, mode);
   else
     hipLaunchKernelGGL(sink_window_attention_kernel<float>, grid, block, lds, stream, (const float*)q, n_heads, n_kv, D,
                        E, (const float*)k_cache, (const float*)v_cache, table, max_pages, page_size, positions,
-                       row_req, window, keep_first, sink, scale, (float*)out, q_start, long_from);
+                       row_req, window, keep_first, sink, scale, (float*)out, q_start, long_from, mode);
   LLMLAB_LAUNCH_CHECK("sink_window_attention");
   return 0;
 }

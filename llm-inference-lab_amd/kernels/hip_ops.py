@@ -23,6 +23,8 @@ from .debug import DispatchRules, KernelDebug
 DT_F32, DT_BF16 = 0, 1
 EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU, EPI_QKV, EPI_PART = 0, 1, 2, 3, 4, 5
 EPI_RELU2 = 6        # STORE through max(z, 0)^2, taken on the float32 sum
+EPI_GEGLU = 7        # the paired product with gelu (tanh form) on the gate instead of silu
+GATE_EPILOGUES = {"silu": EPI_SWIGLU, "gelu_tanh": EPI_GEGLU}
 
 _c_int, _c_long, _c_float, _c_size, _c_ptr = (ctypes.c_int, ctypes.c_long, ctypes.c_float,
                                               ctypes.c_size_t, ctypes.c_void_p)
@@ -497,7 +499,7 @@ class HipOps:
         if x.dtype == torch.bfloat16 and k % 8 != 0:
             raise UnsupportedSizeError(
                 f"bfloat16 matrix products need an inner size that is a multiple of 8, got {k}")
-        want_out = x.dtype if epilogue in (EPI_STORE, EPI_SWIGLU, EPI_RELU2) else torch.float32
+        want_out = x.dtype if epilogue in (EPI_STORE, EPI_SWIGLU, EPI_RELU2, EPI_GEGLU) else torch.float32
         if out.dtype != want_out:
             raise TypeError(f"linear: output must be {want_out}, got {out.dtype}")
         if bias is not None:
@@ -532,12 +534,16 @@ class HipOps:
     def linear_logits(self, x, w, out) -> None:
         self._linear(x, w, out, None, EPI_F32, w.shape[0])
 
-    def linear_swiglu(self, x, w_gate_up, out) -> None:
+    def linear_swiglu(self, x, w_gate_up, out, activation: str = "silu") -> None:
+        """``out = act(x Wg^T) * (x Wu^T)`` with the rows of gate and up interleaved in runs of 16;
+        ``activation``: ``silu`` or ``gelu_tanh``, taken on the float32 sums."""
         inter = out.shape[1]
         if w_gate_up.shape[0] != 2 * ((inter + 15) // 16 * 16):
             raise ValueError(f"linear_swiglu: {w_gate_up.shape[0]} interleaved rows do not belong "
                              f"to {inter} outputs")
-        self._linear(x, w_gate_up, out, None, EPI_SWIGLU, inter)
+        if activation not in GATE_EPILOGUES:
+            raise ValueError(f"linear_swiglu: the gate's activation is one of {sorted(GATE_EPILOGUES)}, got {activation!r}")
+        self._linear(x, w_gate_up, out, None, GATE_EPILOGUES[activation], inter)
 
     # ----------------------------------------------- few rows: fused kernels
     FUSED_MAX_ROWS = 1024         # most rows the few-row kernels take at all
@@ -832,13 +838,14 @@ class HipOps:
             int(page_size), self._ptr(k_cache), self._ptr(v_cache), num_heads, num_kv_heads, head_dim,
             self.num_cus, self._stream())
 
-    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending: Optional[PendingSums] = None) -> None:
+    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending: Optional[PendingSums] = None,
+                          activation: str = "silu") -> None:
         rows, inter = out.shape
         w_gate_up, k = self._fused_common(x, norm_w, w_gate_up, rows)
         self._need(out, "SwiGLU output", torch.bfloat16)
         if x.shape[0] != rows or w_gate_up.shape[0] != 2 * ((inter + 15) // 16 * 16):
             raise ValueError("fused_norm_swiglu: shapes do not fit")
-        self._skinny(x, True, None, norm_w, eps, w_gate_up, None, EPI_SWIGLU, out, rows,
+        self._skinny(x, True, None, norm_w, eps, w_gate_up, None, GATE_EPILOGUES[activation], out, rows,
                      w_gate_up.shape[0], k, out.shape[1], inter, pending=pending)
 
     def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out, pending: Optional[PendingSums] = None) -> None:
@@ -1055,8 +1062,13 @@ class HipOps:
                 lib.llmlab_sink_window_attention.argtypes = [
                     _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                     _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr,
-                    _c_size, _c_int, _c_ptr]
+                    _c_size, _c_int, _c_int, _c_ptr]
                 lib.llmlab_sink_window_attention.restype = _c_int
+                lib.llmlab_project_rotate_write.argtypes = [
+                    _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_float, _c_int,
+                    _c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                    _c_int, _c_ptr]
+                lib.llmlab_project_rotate_write.restype = _c_int
                 lib.llmlab_sink_window_attention_has_mfma.argtypes = [_c_int, _c_int, _c_int, _c_int]
                 lib.llmlab_sink_window_attention_has_mfma.restype = _c_int
                 lib.llmlab_debug_windowed_attention_plain.argtypes = [_c_int]
@@ -1086,6 +1098,11 @@ class HipOps:
                 lib.llmlab_gated_add.restype = _c_int
                 lib.llmlab_softcap.argtypes = [_c_ptr, _c_float, _c_size, _c_ptr]
                 lib.llmlab_softcap.restype = _c_int
+                lib.llmlab_rmsnorm_add.argtypes = [_c_ptr, _c_ptr, _c_int, _c_size, _c_ptr, _c_float, _c_int, _c_int,
+                                                   _c_ptr]
+                lib.llmlab_rmsnorm_add.restype = _c_int
+                lib.llmlab_scaled_sum.argtypes = [_c_ptr, _c_ptr, _c_float, _c_ptr, _c_float, _c_size, _c_ptr]
+                lib.llmlab_scaled_sum.restype = _c_int
             elif kind == "linear_attention":
                 lib.llmlab_gla_decay.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr,
                                                  _c_int, _c_ptr]
@@ -1097,8 +1114,15 @@ class HipOps:
                                                 _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_gla_scan.restype = _c_int
                 lib.llmlab_gla_output.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr,
-                                                  _c_int, _c_int, _c_ptr, _c_int, _c_ptr]
+                                                  _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
                 lib.llmlab_gla_output.restype = _c_int
+                lib.llmlab_delta_gates.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                                                   _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_ptr]
+                lib.llmlab_delta_gates.restype = _c_int
+                lib.llmlab_delta_scan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
+                                                  _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int,
+                                                  _c_ptr]
+                lib.llmlab_delta_scan.restype = _c_int
             elif kind == "routed_experts":
                 lib.llmlab_moe_select.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                                                   _c_ptr, _c_ptr, _c_int, _c_ptr]
@@ -1301,6 +1325,13 @@ class HipOps:
                                        f"channels per head, got {key_dim} and {value_dim}")
         self._mixer_lib("linear_attention")
 
+    def check_delta_rule_sizes(self, num_heads, key_dim, value_dim) -> None:
+        if not 0 < key_dim <= 256 or not 0 < value_dim <= 16384:
+            raise UnsupportedSizeError(f"the delta rule scan keeps a column of the state in a thread's registers: "
+                                       f"up to 256 key channels (and 16384 value channels) per head, got {key_dim} "
+                                       f"and {value_dim}")
+        self._mixer_lib("linear_attention")
+
     def _paged(self, k_cache, v_cache, num_kv_heads, page_size, key_dim, value_dim, dtype):
         pages = k_cache.shape[0]
         if (tuple(k_cache.shape) != (pages, num_kv_heads, page_size, key_dim)
@@ -1370,10 +1401,12 @@ class HipOps:
 
     def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
                               page_size, positions, row_req, window, keep_first, sink, scale, out,
-                              q_start=None, long_from=0, launches=3, max_keys=0) -> None:
+                              q_start=None, long_from=0, launches=3, max_keys=0, weights: str = "softmax") -> None:
         """The query of row ``r`` at position ``i = positions[r]`` of request ``row_req[r]`` attends
         to the cached keys ``j <= i`` with ``i - j < window`` or ``j < keep_first`` (``window`` None:
         all); ``sink`` (float32 per head, or None) adds ``exp(sink)`` to the softmax's denominator.
+        ``weights="sigmoid"``: no softmax; a visible key weighs ``sigmoid(score + sink[h])``
+        (``sink``: then a bias per head on every score, None for none), not normalised over the keys.
         ``long_from > 0`` (``windowed_attention_long_rows``: sizes that the matrix cores take):
         requests that bring at least so many rows (by ``q_start``) are served in tiles of 16 rows
         of a head, the others a row and a group of heads at a time with the row's keys cut into
@@ -1409,7 +1442,61 @@ class HipOps:
                    page_size, self._ptr(positions), self._ptr(row_req), int(window) if window else 0,
                    int(keep_first or 0), self._ptr(sink), float(scale), self._ptr(out),
                    self._ptr(q_start) if long_from else None, int(long_from), int(launches), int(max_keys),
-                   self._ptr(self.workspace), self.workspace.numel(), self.num_cus, self._stream(), lib=lib)
+                   self._ptr(self.workspace), self.workspace.numel(), self.num_cus, self.ATTENTION_WEIGHTS[weights],
+                   self._stream(), lib=lib)
+
+    ATTENTION_WEIGHTS = {"softmax": 0, "sigmoid": 1}
+
+    def project_rotate_write(self, proj, num_heads, num_kv_heads, key_dim, value_dim, bias, freq, rot_dims, magnitude,
+                             mix, mix_weight, v_first, gate_out, q_out, k_cache, v_cache, page_size, positions,
+                             row_req, block_table) -> None:
+        """From the float32 projections ``proj [rows, q | k | v | gates]`` (``bias``, float32 in the same
+        order, is added first): queries and keys with the first ``rot_dims`` channels of every head
+        turned, channel ``2i`` together with ``2i + 1``, by ``positions[r] * freq[i]`` (sine and cosine
+        times ``magnitude``); the queries go to ``q_out``, the keys and the values to the rows' places in
+        the pages.  ``mix``: ``None`` the values as projected; ``"first"`` they are also left, unrounded,
+        in ``v_first [rows, kv heads * value_dim]``; ``"mix"`` ``v <- (1 - mix_weight) v + mix_weight
+        v_first`` before they are stored.  ``gate_out [rows, n]`` float32 (or None) receives the ``n``
+        numbers behind the values."""
+        lib = self._mixer_lib("windowed_attention")
+        self._need(proj, "projections", torch.float32)
+        self._need(q_out, "queries")
+        rows = q_out.shape[0]
+        q_size, k_size, v_size = num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim
+        n_gate = 0 if gate_out is None else gate_out.shape[1]
+        need = q_size + k_size + v_size + n_gate
+        if proj.shape[0] != rows or proj.shape[1] < need or tuple(q_out.shape) != (rows, q_size):
+            raise ValueError(f"project_rotate_write: projections {tuple(proj.shape)}, queries {tuple(q_out.shape)} "
+                             f"do not fit {need} numbers a row")
+        self._paged(k_cache, v_cache, num_kv_heads, page_size, key_dim, value_dim, q_out.dtype)
+        if bias is not None:
+            self._need(bias, "projection bias", torch.float32)
+            if bias.numel() != need:
+                raise ValueError(f"project_rotate_write: a bias of {bias.numel()} numbers for {need} projections")
+        rot_dims = int(rot_dims or 0)
+        if rot_dims:
+            self._need(freq, "rotation frequencies", torch.float32)
+            if rot_dims % 2 or rot_dims > key_dim or freq.numel() != rot_dims // 2:
+                raise ValueError(f"project_rotate_write: {rot_dims} of {key_dim} channels with {freq.numel()} frequencies")
+        code = {None: 0, "first": 1, "mix": 2}[mix]
+        if code:
+            self._need(v_first, "first values", torch.float32)
+            if tuple(v_first.shape) != (rows, v_size):
+                raise ValueError(f"project_rotate_write: first values {tuple(v_first.shape)}, not {(rows, v_size)}")
+        if gate_out is not None:
+            self._need(gate_out, "gates", torch.float32)
+            if gate_out.shape[0] != rows:
+                raise ValueError("project_rotate_write: one row of gates per row")
+        for t, name in ((positions, "positions"), (row_req, "row -> request map"), (block_table, "block table")):
+            self._need(t, name, torch.int32, contiguous=name != "block table")
+        if positions.numel() < rows or row_req.numel() < rows or block_table.stride(1) != 1:
+            raise ValueError("project_rotate_write: one position and one request index per row")
+        self._call(lib.llmlab_project_rotate_write, self._ptr(proj), proj.stride(0), rows, num_heads, num_kv_heads,
+                   key_dim, value_dim, self._ptr(bias), self._ptr(freq) if rot_dims else None, rot_dims,
+                   float(magnitude), code, float(mix_weight or 0.0), self._ptr(v_first) if code else None, n_gate,
+                   self._ptr(gate_out), self._ptr(q_out), self._ptr(k_cache), self._ptr(v_cache), _dt(q_out), page_size,
+                   self._ptr(positions), self._ptr(row_req), self._ptr(block_table), block_table.stride(0),
+                   self._stream(), lib=lib)
 
     def gla_slices(self, key_dim: int) -> int:
         """Into how many pieces the scan leaves each output (one per slice of key channels)."""
@@ -1484,22 +1571,70 @@ class HipOps:
                    self._ptr(chunk_state) if chunk else None, self._ptr(chunk_decay) if chunk else None, max_chunks,
                    self._stream(), lib=lib)
 
-    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out) -> None:
+    OUTPUT_GATES = {"silu": 0, "sigmoid": 1}
+
+    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out, gate: str = "silu") -> None:
         """``out[r, h] = rmsnorm(sum of parts[r, h]) * weight * silu(gate[r, h])`` with the gate at
-        column ``off_gate`` of the float32 ``proj``; ``out`` in the compute dtype."""
+        column ``off_gate`` of the float32 ``proj``; ``out`` in the compute dtype.  ``parts [rows, heads,
+        pieces, value_dim]`` with any number of pieces; ``weight`` of ``value_dim`` numbers (the same for
+        every head) or of ``heads * value_dim``; ``gate="sigmoid"``: ``... * sigmoid(gate[r, h])``."""
         lib = self._mixer_lib("linear_attention")
         self._need(parts, "output pieces", torch.float32)
         self._need(proj, "projections", torch.float32)
         self._need(weight, "output norm weight", torch.float32)
         self._need(out, "mixer output")
         rows = parts.shape[0]
-        if (tuple(parts.shape) != (rows, num_heads, self.gla_slices(key_dim), value_dim) or weight.numel() != value_dim
+        if (parts.dim() != 4 or tuple(parts.shape) != (rows, num_heads, parts.shape[2], value_dim)
+                or weight.numel() not in (value_dim, num_heads * value_dim)
                 or tuple(out.shape) != (rows, num_heads * value_dim) or proj.shape[0] != rows
-                or off_gate < 0 or off_gate + num_heads * value_dim > proj.shape[1]):
+                or off_gate < 0 or off_gate + num_heads * value_dim > proj.shape[1] or gate not in self.OUTPUT_GATES):
             raise ValueError("gla_output: the operands do not fit each other")
+        per_head = 1 if weight.numel() == num_heads * value_dim and num_heads > 1 else 0
         self._call(lib.llmlab_gla_output, self._ptr(parts), rows, num_heads, key_dim, value_dim, self._ptr(weight),
                    float(eps), self._ptr(proj), proj.stride(0), int(off_gate), self._ptr(out), _dt(out),
-                   self._stream(), lib=lib)
+                   int(parts.shape[2]), per_head, self.OUTPUT_GATES[gate], self._stream(), lib=lib)
+
+    def delta_gates(self, proj, off_low, rank, off_rate, w2, w0, rate_bias, decay_scale, decay, rate) -> None:
+        """``decay[r, c] = exp(-decay_scale * sigmoid(w0[c] + w2[c] . tanh(proj[r, off_low : off_low + rank])))``
+        and ``rate[r, c] = sigmoid(proj[r, off_rate + c] + rate_bias[c])``, all float32."""
+        lib = self._mixer_lib("linear_attention")
+        for t, name in ((proj, "projections"), (w2, "decay weight"), (decay, "decays"), (rate, "rates")):
+            self._need(t, name, torch.float32)
+        rows, channels = decay.shape
+        if (proj.shape[0] != rows or tuple(rate.shape) != (rows, channels) or tuple(w2.shape) != (channels, rank)
+                or off_low < 0 or off_low + rank > proj.shape[1] or off_rate < 0 or off_rate + channels > proj.shape[1]):
+            raise ValueError("delta_gates: the operands do not fit each other")
+        for t, name in ((w0, "decay bias"), (rate_bias, "rate bias")):
+            if t is not None:
+                self._need(t, name, torch.float32)
+                if t.numel() != channels:
+                    raise ValueError(f"delta_gates: one {name} per channel")
+        self._call(lib.llmlab_delta_gates, self._ptr(proj), proj.stride(0), rows, int(off_low), int(rank), int(off_rate),
+                   self._ptr(w2), self._ptr(w0), self._ptr(rate_bias), float(decay_scale), self._ptr(decay),
+                   self._ptr(rate), channels, self._stream(), lib=lib)
+
+    def delta_scan(self, proj, off_r, off_k, off_v, decay, rate, num_heads, key_dim, value_dim, key_eps, state, q_start,
+                   req_rows, n_reqs, out) -> None:
+        """The recurrence ``S = diag(decay_t) S - (rate_t * u_t)(u_t^T S) + k_t v_t^T; o_t = S^T r_t`` with
+        ``u_t = k_t / sqrt(|k_t|^2 + key_eps)`` over the rows ``q_start[b] .. q_start[b + 1]`` of each of the
+        step's ``n_reqs`` requests, on the float32 state ``state[req_rows[b]]`` ``[heads, key_dim,
+        value_dim]``, which is left updated; ``out [rows, heads, 1, value_dim]`` float32."""
+        lib = self._mixer_lib("linear_attention")
+        for t, name in ((proj, "projections"), (decay, "decays"), (rate, "rates"), (state, "recurrent state"),
+                        (out, "outputs")):
+            self._need(t, name, torch.float32)
+        self._need(q_start, "request row starts", torch.int32)
+        self._need(req_rows, "state slots", torch.int32)
+        rows = proj.shape[0]
+        if (tuple(decay.shape) != (rows, num_heads * key_dim) or tuple(rate.shape) != tuple(decay.shape)
+                or out.numel() != rows * num_heads * value_dim
+                or tuple(state.shape[1:]) != (num_heads, key_dim, value_dim)
+                or q_start.numel() < n_reqs + 1 or req_rows.numel() < n_reqs or min(off_r, off_k, off_v) < 0
+                or max(off_r + num_heads * key_dim, off_k + num_heads * key_dim, off_v + num_heads * value_dim) > proj.shape[1]):
+            raise ValueError("delta_scan: the operands do not fit each other")
+        self._call(lib.llmlab_delta_scan, self._ptr(proj), proj.stride(0), int(off_r), int(off_k), int(off_v),
+                   self._ptr(decay), self._ptr(rate), num_heads, key_dim, value_dim, float(key_eps), self._ptr(state),
+                   self._ptr(q_start), self._ptr(req_rows), int(n_reqs), self._ptr(out), rows, self._stream(), lib=lib)
 
     # --------------------------------------------------------------- sampling
     # ------------------------------ the stream around sublayers; the latent form of attention
@@ -1634,6 +1769,40 @@ class HipOps:
                 raise ValueError("gated_add: a bias per column of a gate")
         self._call(lib.llmlab_gated_add, self._ptr(x), self._ptr(y), pieces, piece_stride, self._ptr(gate), cols,
                    self._ptr(bias), rows, width, self._stream(), lib=lib)
+
+    def rmsnorm_add(self, y, weight, eps: float, x) -> None:
+        """``x += y / sqrt(mean(y^2) + eps) * weight`` row by row, all float32: the norm of a sublayer's
+        result on its way into the stream.  ``y [rows, width]``, or a product left in pieces
+        (``PendingSums``), which are summed on the way."""
+        lib = self._mixer_lib("stream_ops")
+        self._need(x, "stream", torch.float32)
+        self._need(weight, "norm weight", torch.float32)
+        rows, width = x.shape
+        if isinstance(y, PendingSums):
+            parts, pieces = y.parts, y.splits
+            if (parts.dtype != torch.float32 or parts.dim() != 3 or tuple(parts.shape[1:]) != (rows, width)
+                    or not parts.is_contiguous() or pieces > parts.shape[0]):
+                raise ValueError("rmsnorm_add: pieces are float32 [pieces, rows, width]")
+            stride = parts.stride(0)
+        else:
+            self._need(y, "sublayer result", torch.float32)
+            if tuple(y.shape) != (rows, width):
+                raise ValueError(f"rmsnorm_add: result {tuple(y.shape)} onto a stream {tuple(x.shape)}")
+            parts, pieces, stride = y, 1, 0
+        if weight.numel() != width:
+            raise ValueError("rmsnorm_add: one weight per column")
+        self._call(lib.llmlab_rmsnorm_add, self._ptr(x), self._ptr(parts), int(pieces), int(stride), self._ptr(weight),
+                   float(eps), rows, width, self._stream(), lib=lib)
+
+    def scaled_sum(self, out, y1, a: float, y2, b: float) -> None:
+        """``out = a * y1 + b * y2``, float32 tensors of one shape."""
+        lib = self._mixer_lib("stream_ops")
+        for t, name in ((out, "sum"), (y1, "first term"), (y2, "second term")):
+            self._need(t, name, torch.float32)
+        if tuple(out.shape) != tuple(y1.shape) or tuple(out.shape) != tuple(y2.shape):
+            raise ValueError("scaled_sum: three tensors of one shape")
+        self._call(lib.llmlab_scaled_sum, self._ptr(out), self._ptr(y1), float(a), self._ptr(y2), float(b), out.numel(),
+                   self._stream(), lib=lib)
 
     def softcap(self, x, cap: float) -> None:
         """``x = cap * tanh(x / cap)`` in place, float32."""

@@ -309,19 +309,56 @@ class WindowedSinkAttention(Mixer):
     of the run that the schedule names as its cache (keys as that run stored them, after
     its norm), with its own queries, window and sink.
 
+    ``position``: a position encoding with a ``pair_table()`` (``rope_pairs``) turns queries and keys
+    before the scores are taken; the keys are cached turned.  ``qkv_bias``: the three projections have
+    biases (roles ``q_bias``, ``k_bias``, ``v_bias``), added to the float32 sums.
+    ``weights="sigmoid"``: no softmax; a visible key weighs ``sigmoid(score + b_h)`` with ``b_h`` one
+    learned number per head (role ``score_bias``; ``score_bias=False``: none), and the weights are not
+    normalised over the keys.  ``output_gate="sigmoid"``: one more projection of the layer's input, a
+    single number per head (role ``gate_weight [heads, hidden]``); head ``h``'s output is multiplied
+    by ``sigmoid`` of its number before the output projection.  ``value_mix``: ``"first"`` the layer
+    leaves the values of the step's tokens, unrounded, for later layers; ``"mix"`` its values become
+    ``(1 - lambda) v + lambda v_first`` with ``v_first`` what the ``"first"`` layer left for the same
+    token and ``lambda`` one learned number (role ``value_mix``); the mixed values are what is cached.
+
     Pages: keys ``[kv_heads, P, key_dim]``, values ``[kv_heads, P, value_dim]``."""
 
     writes_output = True
+    WEIGHTS = ("softmax", "sigmoid")
+    VALUE_MIX = (None, "first", "mix")
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int,
                  scale: float, tensors: Dict[str, str], window: Optional[int] = None, keep_first: int = 0,
                  sink: bool = True, qk_norm: Optional[str] = "whole", norm_eps: float = 1e-6,
-                 own_kv: bool = True):
+                 own_kv: bool = True, position: Optional[PartSpec] = None, qkv_bias: bool = False,
+                 weights: str = "softmax", score_bias: bool = False, output_gate: Optional[str] = None,
+                 value_mix: Optional[str] = None):
         super().__init__(tensors)
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if qk_norm not in (None, "whole"):
             raise ValueError(f"qk_norm is None or 'whole', got {qk_norm!r}")
+        if weights not in self.WEIGHTS or value_mix not in self.VALUE_MIX or output_gate not in (None, "sigmoid"):
+            raise ValueError(f"weights is one of {self.WEIGHTS}, value_mix of {self.VALUE_MIX}, output_gate None or "
+                             f"'sigmoid'; got {weights!r}, {value_mix!r}, {output_gate!r}")
+        self.weights, self.value_mix, self.output_gate = weights, value_mix, output_gate
+        self.qkv_bias, self.has_score_bias = bool(qkv_bias), bool(score_bias)
+        self.position = build_part("position", position) if position is not None else None
+        # the projections that turn, carry biases, mix values or gate heads go through one kernel
+        # of their own, which knows no norm over the whole projection and writes keys and values
+        self.rotates = bool(self.position is not None or qkv_bias or value_mix or output_gate)
+        if self.rotates and (qk_norm or not own_kv):
+            raise ValueError("a position encoding, biases, mixed values or an output gate go with keys and values "
+                             "of the layer's own and without a norm over the whole projection")
+        if self.position is not None and not hasattr(self.position, "pair_table"):
+            raise ValueError(f"{type(self.position).__name__} has no pair_table(): this mixer turns neighbouring channels")
+        if weights == "sigmoid" and sink:
+            raise ValueError("a sink belongs to a softmax's denominator; sigmoid weights have none")
+        if score_bias and weights != "sigmoid":
+            raise ValueError("score_bias goes with sigmoid weights")
+        self.w_gate_rows = 0
+        self.b_in = self.score_bias = None
+        self.mix_weight = 0.0
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.key_dim, self.value_dim = int(key_dim), int(value_dim)
         self.scale = float(scale)
@@ -344,7 +381,8 @@ class WindowedSinkAttention(Mixer):
 
     @property
     def in_size(self):
-        return self.q_size + (self.k_size + self.v_size if self.own_kv else 0)
+        return (self.q_size + (self.k_size + self.v_size if self.own_kv else 0)
+                + (self.num_heads if self.output_gate else 0))
 
     def tensor_specs(self):
         t, w = self.tensor_names, self.hidden_size
@@ -353,6 +391,18 @@ class WindowedSinkAttention(Mixer):
         if self.own_kv:
             specs[t["k_weight"]] = TensorSpec((self.k_size, w), MATRIX)
             specs[t["v_weight"]] = TensorSpec((self.v_size, w), MATRIX)
+        if self.qkv_bias:
+            specs[t["q_bias"]] = TensorSpec((self.q_size,), VECTOR)
+            specs[t["k_bias"]] = TensorSpec((self.k_size,), VECTOR)
+            specs[t["v_bias"]] = TensorSpec((self.v_size,), VECTOR)
+        if self.has_score_bias:
+            specs[t["score_bias"]] = TensorSpec((self.num_heads,), VECTOR)
+        if self.output_gate:
+            specs[t["gate_weight"]] = TensorSpec((self.num_heads, w), MATRIX)
+        if self.value_mix and "value_mix" in t:       # (every mixing layer of a model file may carry the number)
+            specs[t["value_mix"]] = TensorSpec((), VECTOR)
+        if self.position is not None:
+            specs.update(self.position.tensor_specs())
         if self.qk_norm:
             specs[t["q_norm"]] = TensorSpec((self.q_size,), VECTOR, INIT_NORM)
             if self.own_kv:
@@ -370,7 +420,20 @@ class WindowedSinkAttention(Mixer):
         rows = [tensors[t["q_weight"]]]
         if self.own_kv:
             rows += [tensors[t["k_weight"]], tensors[t["v_weight"]]]
-        self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())       # one product for q (, k, v)
+        if self.output_gate:
+            rows.append(tensors[t["gate_weight"]])
+        self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())       # one product for q (, k, v, gates)
+        if self.qkv_bias:
+            bias = [tensors[t[r]].float() for r in ("q_bias", "k_bias", "v_bias")]
+            if self.output_gate:
+                bias.append(torch.zeros(self.num_heads, dtype=torch.float32, device=bias[0].device))
+            self.b_in = torch.cat(bias).contiguous()
+        if self.has_score_bias:
+            self.score_bias = tensors[t["score_bias"]].float().contiguous()
+        if self.value_mix == "mix":
+            self.mix_weight = float(tensors[t["value_mix"]].float().reshape(-1)[0])
+        if self.position is not None:
+            self.position.bind(tensors, ops, dtype)
         self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
         if self.qk_norm:
             self.q_norm = tensors[t["q_norm"]].float().contiguous()
@@ -392,10 +455,25 @@ class WindowedSinkAttention(Mixer):
         proj = ctx.scratch("windowed_attention.proj", (rows, self.in_size), torch.float32)
         ops.linear_logits(h, self.w_in, proj)
         q = ctx.scratch("windowed_attention.q", (rows, self.q_size), self.dtype)
-        ops.project_norm_write(proj, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.own_kv,
-                               self.q_norm, self.k_norm, self.norm_eps, q, entry.k_cache, entry.v_cache,
-                               group.page_size, ctx.positions, ctx.row_req, group.block_table)
+        gate = None
+        if self.rotates:
+            freq, rot_dims, magnitude = self.position.pair_table() if self.position is not None else (None, 0, 1.0)
+            if self.output_gate:
+                gate = ctx.scratch("windowed_attention.gate", (rows, self.num_heads), torch.float32)
+            # (every layer that mixes finds the first such layer's values of the step's rows here)
+            first = (ctx.scratch("windowed_attention.first_values", (rows, self.v_size), torch.float32)
+                     if self.value_mix else None)
+            ops.project_rotate_write(proj, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.b_in,
+                                     freq, rot_dims, magnitude, self.value_mix, self.mix_weight, first, gate, q,
+                                     entry.k_cache, entry.v_cache, group.page_size, ctx.positions, ctx.row_req,
+                                     group.block_table)
+        else:
+            ops.project_norm_write(proj, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim, self.own_kv,
+                                   self.q_norm, self.k_norm, self.norm_eps, q, entry.k_cache, entry.v_cache,
+                                   group.page_size, ctx.positions, ctx.row_req, group.block_table)
         mixed = ctx.scratch("windowed_attention.out", (rows, self.num_heads * self.value_dim), self.dtype)
+        sigmoid = self.weights == "sigmoid"
+        kind = dict(weights="sigmoid") if sigmoid else {}
 
         def attend():
             # (which requests bring many rows is read from the step's description when the launch
@@ -403,15 +481,18 @@ class WindowedSinkAttention(Mixer):
             long_from, launches = self._split(ctx, group.page_size)
             ops.sink_window_attention(q, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim,
                                       entry.k_cache, entry.v_cache, group.block_table, group.page_size,
-                                      ctx.positions, ctx.row_req, self.window, self.keep_first, self.sink,
+                                      ctx.positions, ctx.row_req, self.window, self.keep_first,
+                                      self.score_bias if sigmoid else self.sink,
                                       self.scale, mixed, ctx.all_q_start, long_from, launches,
                                       ctx.max_ctx_len if self.window is None
-                                      else min(ctx.max_ctx_len, self.window + self.keep_first))
+                                      else min(ctx.max_ctx_len, self.window + self.keep_first), **kind)
         live = getattr(ops, "live", None)
         if live is not None:
             live(attend)
         else:
             attend()
+        if gate is not None:
+            ops.gate_heads(mixed, gate, self.num_heads, self.value_dim, self.output_gate)
         ops.linear_logits(mixed, self.w_o, out)
 
     def forward(self, h, residual, ctx, entry):
@@ -431,7 +512,7 @@ class WindowedSinkAttention(Mixer):
 
     def weight_bytes(self):
         total = 0
-        for w in (self.w_in, self.w_o, self.q_norm, self.k_norm, self.sink):
+        for w in (self.w_in, self.w_o, self.q_norm, self.k_norm, self.sink, self.b_in, self.score_bias):
             if w is not None:
                 total += w.numel() * w.element_size()
         return total

@@ -149,6 +149,102 @@ class SublayerNormBlock(Block):
         return sum(p.weight_bytes() for p in self.parts())
 
 
+class SandwichNormBlock(Block):
+    """A norm before AND behind each sublayer::
+
+        x += scale1 * post_norm1(mixer(norm1(x)));  x += scale2 * post_norm2(feed_forward(norm2(x)))
+
+    ``scale1`` / ``scale2`` (roles of the block's own tensors, or absent): a learned vector that
+    multiplies the normed result element by element (a layer scale); it is folded into the
+    post-norm's weight when the block is bound.  The post-norms are RMS norms (anything with
+    ``rms_params()``); they act on the sublayer's float32 result, and norm, product and sum are
+    float32.  A block without a feed-forward has the first half only."""
+
+    def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, post_norm1: PartSpec,
+                 norm2: PartSpec = None, feed_forward: PartSpec = None, post_norm2: PartSpec = None,
+                 tensors: Dict[str, str] = None):
+        super().__init__(tensors)
+        if len({feed_forward is None, norm2 is None, post_norm2 is None}) != 1:
+            raise ValueError("a feed-forward and its two norms come together")
+        self.hidden_size = int(hidden_size)
+        self.norm1 = build_part("norm", norm1)
+        self.mixer = build_part("mixer", mixer)
+        self.post_norm1 = build_part("norm", post_norm1)
+        self.norm2 = build_part("norm", norm2) if norm2 is not None else None
+        self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
+        self.post_norm2 = build_part("norm", post_norm2) if post_norm2 is not None else None
+        self.post = [None, None]       # (weight with the layer scale folded in, eps) of each half
+
+    def parts(self):
+        return [p for p in (self.norm1, self.mixer, self.post_norm1, self.norm2, self.feed_forward, self.post_norm2)
+                if p is not None]
+
+    def mixer_part(self):
+        return self.mixer
+
+    def tensor_specs(self):
+        specs = {}
+        for p in self.parts():
+            specs.update(p.tensor_specs())
+        for role in ("scale1", "scale2"):
+            if role in self.tensor_names and (role == "scale1" or self.feed_forward is not None):
+                specs[self.tensor_names[role]] = TensorSpec((self.hidden_size,), VECTOR)
+        return specs
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        for p in self.parts():
+            p.bind(tensors, ops, dtype)
+        for i, norm in enumerate((self.post_norm1, self.post_norm2)):
+            if norm is None:
+                continue
+            params = norm.rms_params() if hasattr(norm, "rms_params") else None
+            if params is None:
+                raise ValueError(f"{type(norm).__name__} is no RMS norm: the norm behind a sublayer is one")
+            weight = params[0].float()
+            role = f"scale{i + 1}"
+            if role in self.tensor_names:
+                weight = weight * tensors[self.tensor_names[role]].float()
+            self.post[i] = (weight.contiguous(), float(params[1]))
+
+    def kernel_libraries(self):
+        return [("stream_ops", None)] + super().kernel_libraries()
+
+    def _fold(self, residual, ctx):
+        pending = getattr(ctx, "pending", None)
+        if pending is not None:
+            self.ops.add_pending(residual, pending)
+            ctx.pending = None
+
+    def _half(self, i, norm, part, residual, ctx, *view):
+        ops, rows = self.ops, residual.shape[0]
+        self._fold(residual, ctx)
+        h = ctx.scratch("block.normed", (rows, self.hidden_size), self.dtype)
+        norm.forward(residual, h)
+        y = ctx.scratch("block.sublayer_out", (rows, self.hidden_size), torch.float32)
+        if part.writes_output:
+            part.forward_into(h, y, ctx, *view)
+        elif hasattr(part, "forward_pending"):
+            pieces = part.forward_pending(h, y, ctx, *view)      # (a product left in pieces is summed by the norm)
+            if pieces is not None:
+                y = pieces
+        else:
+            ops.activation(y, y, "zero")
+            part.forward(h, y, ctx, *view)
+            self._fold(y, ctx)
+        weight, eps = self.post[i]
+        ops.rmsnorm_add(y, weight, eps, residual)
+
+    def forward(self, residual, ctx, entry):
+        self._half(0, self.norm1, self.mixer, residual, ctx, entry)
+        if self.feed_forward is not None:
+            self._half(1, self.norm2, self.feed_forward, residual, ctx)
+
+    def weight_bytes(self):
+        own = sum(w.numel() * w.element_size() for w, _ in (p for p in self.post if p is not None))
+        return own + sum(p.weight_bytes() for p in self.parts())
+
+
 class GatedConvBlock(Block):
     """A pre-norm layer whose sublayers read their input through a short causal convolution and
     whose results pass a gate before they are summed::
@@ -428,5 +524,6 @@ register_part("block", "prenorm", PreNormBlock)
 register_part("block", "gated_conv", GatedConvBlock)
 register_part("embedding", "pair_hash_embedding", PairHashEmbedding)
 register_part("block", "sublayer_norm", SublayerNormBlock)
+register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "linear_head", LinearHead)

@@ -54,13 +54,19 @@ class SwiGLU(FeedForward):
     exp(-z))``; accumulators, the sigmoid and the product in float32.
 
     Formula: rust/engine/src/runner/model/qwen2/engine.rs:1234-1294,
-    rust/engine/src/runner/model/qwen2/kernels.rs:1469-1486."""
+    rust/engine/src/runner/model/qwen2/kernels.rs:1469-1486.
+
+    ``activation="gelu_tanh"``: the gate goes through ``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715
+    z^3)))`` instead of ``silu``; everything else stays."""
+
+    ACTIVATIONS = ("silu", "gelu_tanh")
 
     def __init__(self, hidden_size: int, intermediate_size: int, tensors: Dict[str, str],
                  activation: str = "silu"):
         super().__init__(tensors)
-        if activation != "silu":
-            raise ValueError(f"SwiGLU supports activation 'silu', got '{activation}'")
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"a gated feed-forward takes the activations {self.ACTIVATIONS}, got '{activation}'")
+        self.activation = activation
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         # the kernels' inner sizes are multiples of 8: an intermediate size that is not is laid out
@@ -87,6 +93,13 @@ class SwiGLU(FeedForward):
     takes_normed_input = True
     keeps_launches = True
 
+    def _act(self):
+        """(silu is what the kernels do when they are told nothing)"""
+        return () if self.activation == "silu" else (self.activation,)
+
+    def _act_kw(self):
+        return {} if self.activation == "silu" else dict(activation=self.activation)
+
     def forward_pending(self, h, out, ctx):
         """The result into ``out`` (float32), or, where the down product is left in pieces, the
         pieces themselves (``PendingSums``; ``out`` is not written): for a caller that does
@@ -95,7 +108,7 @@ class SwiGLU(FeedForward):
         if isinstance(h, NormedInput):
             h = h.tensor()
         act = ctx.scratch("swiglu.act", (rows, self.kernel_size), self.dtype)
-        self.ops.linear_swiglu(h, self.w_gate_up, act)
+        self.ops.linear_swiglu(h, self.w_gate_up, act, *self._act())
         splits = self.ops.split_count(rows, self.dtype, self.hidden_size, self.kernel_size)
         if splits > 1:
             parts = ctx.scratch("swiglu.pieces", (splits, rows, self.hidden_size), torch.float32)
@@ -110,11 +123,11 @@ class SwiGLU(FeedForward):
                                                                  self.w_gate_up.shape[0])
         rms = h.rms() if fuse else None      # (folds pieces still owed to the stream; else the norm does)
         if rms is not None:
-            self.ops.fused_norm_swiglu(rms[0], rms[2], rms[3], self.w_gate_up, act)
+            self.ops.fused_norm_swiglu(rms[0], rms[2], rms[3], self.w_gate_up, act, **self._act_kw())
         else:
             if isinstance(h, NormedInput):
                 h = h.tensor()
-            self.ops.linear_swiglu(h, self.w_gate_up, act)
+            self.ops.linear_swiglu(h, self.w_gate_up, act, *self._act())
         splits = self.ops.split_count(rows, self.dtype, self.hidden_size, self.kernel_size)
         if splits > 1 and hasattr(ctx, "pending") and ctx.pending is None:
             # a narrow output: the product is cut along the inner size so that it spreads

@@ -151,4 +151,146 @@ class GatedLinearAttention(Mixer):
                    for w in (self.w_in, self.w_o, self.w_decay, self.b_decay, self.norm_weight) if w is not None)
 
 
+class DeltaRuleAttention(Mixer):
+    """A recurrent mixer whose matrix-valued state forgets along the current key before it
+    learns the new pair (a generalised delta rule).
+
+    With ``D = key_dim`` and ``E = value_dim`` (default ``D``): ``r = Wr h``, ``k = Wk h`` (``heads x
+    D``), ``v = Wv h`` (``heads x E``); decays ``w = exp(-decay_scale * sigmoid(W2 tanh(W1 h) + w0))``
+    and removal rates ``a = sigmoid(Wa h + ba)``, both per head and key channel; per head, token by
+    token, with the unit key ``u = k / sqrt(|k|^2 + key_eps)``::
+
+        S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T     (S is D x E; both terms
+        o_t = S_t^T r_t                                                        read the old state)
+
+    then every head's ``o_t`` is divided by its root mean square over ``E`` (``norm_eps`` inside the
+    root), the heads are put side by side, multiplied by a weight of all heads' size and by
+    ``sigmoid(Wg h)`` (``gate="silu"``: by ``silu``), and projected by ``Wo``.
+
+    The state lives in float32 in one slot per request (``state_spec``), zero at a sequence's
+    start, and is carried from step to step; decays, rates, the unit key, the recurrence and the
+    norm are float32 throughout, and the projections reach them unrounded (the 32-bit sums of the
+    matrix products).  ``decay_rank`` None: the rank of the decay projection is whatever the model
+    file's tensors have.
+
+    Tensor roles: ``r_weight, k_weight, v_weight, gate_weight, rate_weight, rate_bias, decay_down,
+    decay_up, decay_bias, out_norm, o_weight``."""
+
+    writes_output = True
+    keeps_launches = True
+    DEFAULT_DECAY_SCALE = 0.6065306597126334      # exp(-1/2)
+
+    def __init__(self, hidden_size: int, num_heads: int, key_dim: int, tensors: Dict[str, str],
+                 value_dim: Optional[int] = None, decay_rank: Optional[int] = None,
+                 decay_scale: float = DEFAULT_DECAY_SCALE, key_eps: float = 1e-6, norm_eps: float = 1e-6,
+                 gate: str = "sigmoid"):
+        super().__init__(tensors)
+        self.hidden_size, self.num_heads, self.key_dim = int(hidden_size), int(num_heads), int(key_dim)
+        self.value_dim = self.key_dim if value_dim is None else int(value_dim)
+        self.decay_rank = None if decay_rank is None else int(decay_rank)
+        self.decay_scale, self.key_eps, self.norm_eps = float(decay_scale), float(key_eps), float(norm_eps)
+        if gate not in ("sigmoid", "silu"):
+            raise ValueError(f"the output gate is 'sigmoid' or 'silu', got {gate!r}")
+        self.gate = gate
+        self.w_in = self.w_o = self.w_decay = self.b_decay = self.b_rate = self.norm_weight = None
+        self.offsets = {}
+        self.in_size = 0
+
+    @property
+    def qk_size(self):
+        return self.num_heads * self.key_dim
+
+    @property
+    def v_size(self):
+        return self.num_heads * self.value_dim
+
+    def tensor_specs(self):
+        t, w = self.tensor_names, self.hidden_size
+        return {
+            t["r_weight"]: TensorSpec((self.qk_size, w), MATRIX),
+            t["k_weight"]: TensorSpec((self.qk_size, w), MATRIX),
+            t["v_weight"]: TensorSpec((self.v_size, w), MATRIX),
+            t["gate_weight"]: TensorSpec((self.v_size, w), MATRIX),
+            t["rate_weight"]: TensorSpec((self.qk_size, w), MATRIX),
+            t["rate_bias"]: TensorSpec((self.qk_size,), VECTOR),
+            t["decay_down"]: TensorSpec((self.decay_rank, w), MATRIX),
+            t["decay_up"]: TensorSpec((self.qk_size, self.decay_rank), MATRIX),
+            t["decay_bias"]: TensorSpec((self.qk_size,), VECTOR),
+            t["out_norm"]: TensorSpec((self.v_size,), VECTOR, INIT_NORM),
+            t["o_weight"]: TensorSpec((w, self.v_size), MATRIX),
+        }
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        ops.check_delta_rule_sizes(self.num_heads, self.key_dim, self.value_dim)
+        ops.check_product_sizes(self.hidden_size, dtype, "delta rule projections (hidden size)")
+        ops.check_product_sizes(self.v_size, dtype, "delta rule output projection (heads * value size)")
+        t = self.tensor_names
+        rank = int(tensors[t["decay_down"]].shape[0])
+        if int(tensors[t["decay_up"]].shape[1]) != rank:
+            raise ValueError(f"{t['decay_down']} has {rank} rows but {t['decay_up']} has "
+                             f"{int(tensors[t['decay_up']].shape[1])} columns: the two factors of the decay "
+                             f"projection do not fit")
+        self.decay_rank = rank
+        # one product for r, k, v, the gate, the rates and the low-rank input of the decays
+        self.offsets, at, rows = {}, 0, []
+        for role in ("r_weight", "k_weight", "v_weight", "gate_weight", "rate_weight", "decay_down"):
+            self.offsets[role] = at
+            rows.append(tensors[t[role]])
+            at += rows[-1].shape[0]
+        self.in_size = at
+        self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())
+        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
+        # the second factor of the decays is applied in float32, inside the gates' kernel
+        self.w_decay = tensors[t["decay_up"]].float().contiguous()
+        self.b_decay = tensors[t["decay_bias"]].float().contiguous()
+        self.b_rate = tensors[t["rate_bias"]].float().contiguous()
+        self.norm_weight = tensors[t["out_norm"]].float().contiguous()
+
+    def state_spec(self):
+        return {"s": ((self.num_heads, self.key_dim, self.value_dim), torch.float32)}
+
+    def forward_into(self, h, out, ctx, entry):
+        ops, rows, o = self.ops, h.shape[0], self.offsets
+        proj = ctx.scratch("delta_rule.proj", (rows, self.in_size), torch.float32)
+        ops.linear_logits(h, self.w_in, proj)
+        decay = ctx.scratch("delta_rule.decay", (rows, self.qk_size), torch.float32)
+        rate = ctx.scratch("delta_rule.rate", (rows, self.qk_size), torch.float32)
+        ops.delta_gates(proj, o["decay_down"], self.decay_rank, o["rate_weight"], self.w_decay, self.b_decay,
+                        self.b_rate, self.decay_scale, decay, rate)
+        outs = ctx.scratch("delta_rule.outputs", (rows, self.num_heads, 1, self.value_dim), torch.float32)
+        state = entry.state["s"]
+
+        def scan():
+            # (how many requests the step has is read when the launch is made, also when it is made
+            # again from a kept sequence of calls)
+            ops.delta_scan(proj, o["r_weight"], o["k_weight"], o["v_weight"], decay, rate, self.num_heads,
+                           self.key_dim, self.value_dim, self.key_eps, state, ctx.all_q_start, ctx.all_req_rows,
+                           ctx.n_reqs, outs)
+        live = getattr(ops, "live", None)
+        if live is not None:
+            live(scan)
+        else:
+            scan()
+        mixed = ctx.scratch("delta_rule.out", (rows, self.v_size), self.dtype)
+        ops.gla_output(outs, self.num_heads, self.key_dim, self.value_dim, self.norm_weight, self.norm_eps, proj,
+                       o["gate_weight"], mixed, self.gate)
+        ops.linear_logits(mixed, self.w_o, out)
+
+    def forward(self, h, residual, ctx, entry):
+        if isinstance(h, NormedInput):
+            h = h.tensor()
+        y = ctx.scratch("delta_rule.sum", (1,) + tuple(residual.shape), torch.float32)
+        self.forward_into(h, y[0], ctx, entry)
+        self.ops.add_pending(residual, PendingSums(y, 1))
+
+    def kernel_libraries(self):
+        return [("linear_attention", None)]
+
+    def weight_bytes(self):
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o, self.w_decay, self.b_decay, self.b_rate,
+                                                          self.norm_weight) if w is not None)
+
+
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+register_part("mixer", "delta_rule_attention", DeltaRuleAttention)

@@ -69,6 +69,72 @@ class RotaryEmbedding(PositionEncoding):
         self.ops.rope_inplace(k, positions, self.inv_freq)
 
 
+class PairRotary(PositionEncoding):
+    """Rotation of neighbouring channels: of the first ``rotary_dim`` channels of a head, channel
+    ``2i`` turns together with channel ``2i + 1`` by the angle ``position * f_i``, ``(u, v) -> (u cos
+    - v sin, v cos + u sin)`` with ``f_i = theta^(-2i/rotary_dim)``; the other channels pass.  Angles,
+    sines and cosines are float32.
+
+    ``scaling`` (``factor, original, fast, slow``) stretches the slow frequencies for sequences longer
+    than the ``original`` length: with ``n(t) = rotary_dim ln(original / (2 pi t)) / (2 ln theta)`` (the
+    pair whose wave turns ``t`` times over the original length), ``lo = max(floor(n(fast)), 0)``, ``hi
+    = min(ceil(n(slow)), rotary_dim - 1)`` and ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``
+    the frequency becomes ``f_i / factor * ramp_i + f_i (1 - ramp_i)``, and sines and cosines are
+    multiplied by ``magnitude_slope * ln(factor) + 1``.
+
+    Mixers that take this part ask for ``pair_table()``: the frequencies, how many channels turn,
+    and the magnitude."""
+
+    keeps_launches = True
+
+    def __init__(self, dim: int, theta: float, tensors: Optional[Dict[str, str]] = None,
+                 rotary_dim: Optional[int] = None, scaling: Optional[Dict[str, float]] = None,
+                 magnitude_slope: float = 0.1):
+        super().__init__(tensors)
+        self.dim = int(dim)
+        self.rotary_dim = self.dim if rotary_dim is None else int(rotary_dim)
+        if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.dim:
+            raise ValueError(f"a head of {dim} channels of which {self.rotary_dim} turn in pairs")
+        self.theta = float(theta)
+        self.scaling = dict(scaling) if scaling else None
+        if self.scaling is not None:
+            missing = [k for k in ("factor", "original", "fast", "slow") if k not in self.scaling]
+            if missing:
+                raise ValueError(f"frequency scaling needs {missing}")
+        self.magnitude_slope = float(magnitude_slope)
+        self.freq: Optional[torch.Tensor] = None
+        self.magnitude = 1.0
+
+    def frequencies(self):
+        """``(f [rotary_dim / 2] as Python floats, magnitude)``, worked out in double precision."""
+        import math
+        n = self.rotary_dim
+        f = [self.theta ** (-2.0 * i / n) for i in range(n // 2)]
+        sc = self.scaling
+        if sc is None:
+            return f, 1.0
+        factor, original = float(sc["factor"]), float(sc["original"])
+
+        def pair_of(turns):
+            return n * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+        lo = max(math.floor(pair_of(float(sc["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(sc["slow"]))), n - 1)
+        span = max(hi - lo, 0.001)
+        out = []
+        for i, fi in enumerate(f):
+            ramp = min(max((i - lo) / span, 0.0), 1.0)
+            out.append(fi / factor * ramp + fi * (1.0 - ramp))
+        return out, self.magnitude_slope * math.log(factor) + 1.0
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        f, self.magnitude = self.frequencies()
+        self.freq = torch.tensor(f, dtype=torch.float64).to(torch.float32).to(ops.device)
+
+    def pair_table(self):
+        return self.freq, self.rotary_dim, self.magnitude
+
+
 class NoPosition(PositionEncoding):
     """No position encoding: queries and keys are used as projected."""
 
@@ -82,4 +148,5 @@ class NoPosition(PositionEncoding):
 
 
 register_part("position", "rope", RotaryEmbedding)
+register_part("position", "rope_pairs", PairRotary)
 register_part("position", "none", NoPosition)

@@ -61,7 +61,8 @@ class EmuOps:
                 "paged_attention", "argmax", "sample", "layernorm", "layernorm_add", "activation",
                 "project_norm_write", "sink_window_attention", "gla_decay", "gla_scan", "gla_output",
                 "gate_heads", "add_row_vector", "moe_select", "moe_add_chosen", "embed_pairs", "causal_conv", "norm_conv",
-                "gated_add", "latent_norm_write", "head_products", "softcap")
+                "gated_add", "latent_norm_write", "head_products", "softcap", "project_rotate_write", "delta_gates",
+                "delta_scan", "rmsnorm_add", "scaled_sum")
 
     def __init__(self, device="cpu", fuse=True):
         self.device = torch.device(device)
@@ -219,7 +220,7 @@ class EmuOps:
         self._count("linear_logits")
         out.copy_(x.float() @ w.float().t())
 
-    def linear_swiglu(self, x, w_gu, out):
+    def linear_swiglu(self, x, w_gu, out, activation="silu"):
         """w_gu rows alternate in runs of 16: gate rows of 16 outputs, then the
         up rows of the same outputs."""
         self._count("linear_swiglu")
@@ -228,7 +229,11 @@ class EmuOps:
         y = y.view(x.shape[0], -1, 2, 16)
         gate = y[:, :, 0, :].reshape(x.shape[0], -1)[:, :inter]
         up = y[:, :, 1, :].reshape(x.shape[0], -1)[:, :inter]
-        out.copy_((gate / (1.0 + torch.exp(-gate)) * up).to(out.dtype))
+        if activation == "gelu_tanh":
+            act = 0.5 * gate * (1.0 + torch.tanh(0.7978845608028654 * (gate + 0.044715 * gate ** 3)))
+        else:
+            act = gate / (1.0 + torch.exp(-gate))
+        out.copy_((act * up).to(out.dtype))
 
     # ------------------------------------------- layer norm, plain activations
     @staticmethod
@@ -284,7 +289,7 @@ class EmuOps:
 
     def sink_window_attention(self, q, num_heads, num_kv_heads, key_dim, value_dim, k_cache, v_cache, block_table,
                               page_size, positions, row_req, window, keep_first, sink, scale, out,
-                              q_start=None, long_from=0, launches=3, max_keys=0):
+                              q_start=None, long_from=0, launches=3, max_keys=0, weights="softmax"):
         """(``long_from``, ``launches``: how the kernels share the rows; the result is the same.)"""
         self._count("sink_window_attention")
         rows = q.shape[0]
@@ -300,10 +305,94 @@ class EmuOps:
             v = cache_layout.value_quads(v_cache)[pages, :, offs >> 2, :, offs & 3].float()
             for h in range(num_heads):
                 s = (k[:, h // group] @ qf[r, h]) * scale
+                if weights == "sigmoid":
+                    w = torch.sigmoid(s + (sink[h].float() if sink is not None else 0.0))
+                    if out.dtype != torch.float32:      # (the matrix cores take the weights rounded)
+                        w = w.to(out.dtype).float()
+                    out[r, h * value_dim:(h + 1) * value_dim] = (w @ v[:, h // group]).to(out.dtype)
+                    continue
                 if sink is not None:
                     s = torch.cat([s, sink[h].float().view(1)])
                 w = torch.softmax(s, 0)[:len(js)]
                 out[r, h * value_dim:(h + 1) * value_dim] = (w @ v[:, h // group]).to(out.dtype)
+
+    def project_rotate_write(self, proj, num_heads, num_kv_heads, key_dim, value_dim, bias, freq, rot_dims, magnitude,
+                             mix, mix_weight, v_first, gate_out, q_out, k_cache, v_cache, page_size, positions,
+                             row_req, block_table):
+        self._count("project_rotate_write")
+        rows = q_out.shape[0]
+        qs, ks, vs = num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim
+        p = proj.float()[:, :qs + ks + vs + (0 if gate_out is None else gate_out.shape[1])]
+        if bias is not None:
+            p = p + bias.float()
+        pos = positions[:rows].float()
+
+        def turned(x, heads):
+            x = x.reshape(rows, heads, key_dim).clone()
+            if rot_dims:
+                ang = pos.unsqueeze(-1) * freq.float()                       # float32 angles
+                cos, sin = (torch.cos(ang) * magnitude).unsqueeze(1), (torch.sin(ang) * magnitude).unsqueeze(1)
+                u, v = x[..., 0:rot_dims:2].clone(), x[..., 1:rot_dims:2].clone()
+                x[..., 0:rot_dims:2] = u * cos - v * sin
+                x[..., 1:rot_dims:2] = v * cos + u * sin
+            return x
+        q_out.copy_(turned(p[:, :qs], num_heads).reshape(rows, qs).to(q_out.dtype))
+        k = turned(p[:, qs:qs + ks], num_kv_heads).to(k_cache.dtype)
+        v = p[:, qs + ks:qs + ks + vs]
+        if mix == "first":
+            v_first.copy_(v)
+        elif mix == "mix":
+            v = (1.0 - mix_weight) * v + mix_weight * v_first
+        v = v.to(v_cache.dtype).view(rows, num_kv_heads, value_dim)
+        if gate_out is not None:
+            gate_out.copy_(p[:, qs + ks + vs:])
+        for r in range(rows):
+            at = int(positions[r])
+            page = int(block_table[int(row_req[r]), at // page_size])
+            o = at % page_size
+            k_cache[page, :, o] = k[r]
+            cache_layout.value_quads(v_cache[page])[:, o >> 2, :, o & 3] = v[r]
+
+    def check_delta_rule_sizes(self, num_heads, key_dim, value_dim):
+        pass
+
+    def delta_gates(self, proj, off_low, rank, off_rate, w2, w0, rate_bias, decay_scale, decay, rate):
+        self._count("delta_gates")
+        z = torch.tanh(proj[:, off_low:off_low + rank].float()) @ w2.float().t()
+        if w0 is not None:
+            z = z + w0.float()
+        decay.copy_(torch.exp(-decay_scale * torch.sigmoid(z)))
+        za = proj[:, off_rate:off_rate + decay.shape[1]].float()
+        if rate_bias is not None:
+            za = za + rate_bias.float()
+        rate.copy_(torch.sigmoid(za))
+
+    def delta_scan(self, proj, off_r, off_k, off_v, decay, rate, num_heads, key_dim, value_dim, key_eps, state, q_start,
+                   req_rows, n_reqs, out):
+        self._count("delta_scan")
+        H, D, E = num_heads, key_dim, value_dim
+        o = out.view(-1, H, E)
+        for b in range(n_reqs):
+            st = state[int(req_rows[b])]
+            for t in range(int(q_start[b]), int(q_start[b + 1])):
+                r = proj[t, off_r:off_r + H * D].view(H, D)
+                k = proj[t, off_k:off_k + H * D].view(H, D)
+                v = proj[t, off_v:off_v + H * E].view(H, E)
+                u = k / torch.sqrt((k * k).sum(-1, keepdim=True) + key_eps)
+                dot = torch.einsum("hd,hde->he", u, st)
+                new = (decay[t].view(H, D, 1) * st - (rate[t].view(H, D) * u).unsqueeze(-1) * dot.unsqueeze(-2)
+                       + k.unsqueeze(-1) * v.unsqueeze(-2))
+                st.copy_(new)
+                o[t] = torch.einsum("hde,hd->he", st, r)
+
+    def rmsnorm_add(self, y, weight, eps, x):
+        self._count("rmsnorm_add")
+        v = self._owed(y) if isinstance(y, PendingSums) else y.float()
+        x.add_(v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight.float())
+
+    def scaled_sum(self, out, y1, a, y2, b):
+        self._count("scaled_sum")
+        out.copy_(a * y1 + b * y2)
 
     SCAN_SLICE = 16
 
@@ -339,12 +428,13 @@ class EmuOps:
                 for s in range(parts.shape[2]):
                     parts[t, :, s] = o[:, s * S:(s + 1) * S].sum(1)
 
-    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out):
+    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out, gate="silu"):
         self._count("gla_output")
         o = parts.sum(2)                                        # [rows, H, E]
-        y = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * weight.float()
+        w = weight.float().view(num_heads, value_dim) if weight.numel() == num_heads * value_dim else weight.float()
+        y = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * w
         g = proj[:, off_gate:off_gate + num_heads * value_dim].float().view(-1, num_heads, value_dim)
-        out.copy_((y * g * torch.sigmoid(g)).reshape(out.shape).to(out.dtype))
+        out.copy_((y * (g if gate == "silu" else 1.0) * torch.sigmoid(g)).reshape(out.shape).to(out.dtype))
 
     # ------------------------------------------------- fused few-row kernels
     FUSED_MAX_ROWS = 64
@@ -578,10 +668,10 @@ class EmuOps:
                            block_table, page_size, k_cache, v_cache)
         q_out.copy_(qkv[:, :num_heads * head_dim].to(q_out.dtype))
 
-    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending=None):
+    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending=None, activation="silu"):
         self._count("fused_norm_swiglu")
         h = self._normed(x, None, norm_w, eps, x.shape[0], pending)
-        self.linear_swiglu(h, w_gate_up, out)
+        self.linear_swiglu(h, w_gate_up, out, activation)
 
     def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out, pending=None):
         self._count("fused_norm_logits")
