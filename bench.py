@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S]
                     [--shape 0.5b|7b|32b] [--layers L] [--dtype bf16|f32]
     python bench.py --mixed [--shape 7b] [--requests 64] [--chunk 512] [--outputs 64]
-    python bench.py --design vivevik|ruvalorn|minodra [--size small|medium|large] [--context 2048]
+    python bench.py --design vivevik|ruvalorn|minodra|ninisun [--size small|medium|large] [--context 2048]
 
 Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
 batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
@@ -47,6 +47,12 @@ keys, a gate per head, mixtures of experts behind a grouped router, some layers 
 ``--design minodra``: the same for the Minodra design (attention over one cached latent vector per
 token, a short convolution in front of every sublayer, gated sums into the stream, mixtures of
 squared-ReLU experts behind a sigmoid router in every other layer).
+
+``--design ninisun``: the same for the Ninisun design (norms on both sides of every sublayer, windowed
+attention with turned neighbouring channels and values mixed with the first layer's, every third
+layer attention with sigmoid weights beside a delta-rule state, gelu-gated feed-forwards), beside
+the Vivevik design of equal size (the closest one: the same attention kernels, a recurrent layer in
+every three) and the Qwen2 decoder.
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -242,6 +248,51 @@ def minodra_flops(cfg, tokens):
     return total + 2 * w * cfg.vocab
 
 
+# ``--design ninisun``: layers in threes like Vivevik's: a parallel layer (attention with sigmoid
+# weights over all positions beside a delta-rule state of 64 x 64 numbers per head, width / 64
+# heads), then two windowed attention layers whose values are mixed with the first one's; half of
+# every head turns; every layer has the gated feed-forward.
+def ninisun_config(size):
+    import llm_inference_lab_amd as lab
+    width, heads, kv, dim, ff, layers = DESIGN_SIZES[size]
+    listed = []
+    for i in range(layers):
+        if i % 3 == 0:
+            left = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5,
+                        rot=dict(dims=dim // 2, base=1e6, scaling=dict(factor=4.0, original=1024, fast=32.0, slow=1.0)))
+            mixer = dict(left=left, right=dict(heads=width // 64, dim=64), left_scale=0.8, right_scale=0.9)
+            listed.append(dict(type="parallel", mixer=mixer, mlp=dict(kind="dense", ff=ff)))
+        else:
+            mixer = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5, v_mix=True,
+                         rot=dict(dims=dim // 2, base=5e5), mask=dict(size=DESIGN_WINDOW, keep_first=DESIGN_KEEP))
+            listed.append(dict(type="attention", mixer=mixer, mlp=dict(kind="dense", ff=ff)))
+    return lab.NinisunConfig.from_dict(dict(architecture="Ninisun", vocab=DESIGN_VOCAB, width=width,
+                                            norm=dict(eps=1e-6), layers=listed))
+
+
+def ninisun_flops(cfg, tokens):
+    """Multiply-adds times two of one prompt of ``tokens`` positions (products and attention; the
+    recurrence counts its removal, its update and its read-out: three passes over the state)."""
+    w, total = cfg.width, 0
+    rank = cfg.DEFAULT_DECAY_RANK
+    for l in cfg.layers:
+        for a, window in ((l.attention, True), (l.left, False)):
+            if a is None:
+                continue
+            q, k, v = a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim
+            total += tokens * 2 * (w * (q + k + v) + a.heads * a.vdim * w)
+            size = (a.window or tokens) if window else tokens
+            seen = sum(min(i + 1, size + a.keep_first) for i in range(tokens))
+            total += 2 * seen * a.heads * (a.dim + a.vdim)
+        if l.right is not None:
+            n = l.right.heads * l.right.dim
+            total += tokens * 2 * (w * (5 * n + rank) + rank * n + n * w)
+            total += tokens * 6 * l.right.heads * l.right.dim * l.right.dim
+        if l.mlp is not None:
+            total += tokens * 6 * w * l.mlp.ff
+    return total + 2 * w * cfg.vocab
+
+
 def design_run(args, bracket=None):
     """``--design vivevik``: both models at each size, one after the other on the same GPU.
     ``--only-model``, ``--only-prefill`` / ``--only-decode`` and ``--batch`` narrow the run (for
@@ -261,8 +312,12 @@ def design_run(args, bracket=None):
                                               num_key_value_heads=kv, head_dim=dim, tie_word_embeddings=True))
         record[size] = {"width": width, "heads": heads, "kv_heads": kv, "head_dim": dim, "ff": ff, "layers": layers,
                         "context": context, "window": DESIGN_WINDOW}
-        design = {"ruvalorn": ruvalorn_config, "minodra": minodra_config, "vivevik": vivevik_config}[args.design](size)
-        for label, cfg in ((args.design, design), ("qwen2", qwen)):
+        design = {"ruvalorn": ruvalorn_config, "minodra": minodra_config, "vivevik": vivevik_config,
+                  "ninisun": ninisun_config}[args.design](size)
+        beside = [("qwen2", qwen)]
+        if args.design == "ninisun":         # (the closest design first)
+            beside.insert(0, ("vivevik", vivevik_config(size)))
+        for label, cfg in [(args.design, design)] + beside:
             if args.only_model and label != args.only_model:
                 continue
             expected = CausalLM(get_architecture(cfg.architecture).build_spec(cfg)).tensor_specs()
@@ -279,6 +334,7 @@ def design_run(args, bracket=None):
             flops = (vivevik_flops(cfg, args.prefill_tokens) if label == "vivevik" else
                      ruvalorn_flops(cfg, args.prefill_tokens) if label == "ruvalorn" else
                      minodra_flops(cfg, args.prefill_tokens) if label == "minodra" else
+                     ninisun_flops(cfg, args.prefill_tokens) if label == "ninisun" else
                      prefill_flops(cfg, args.prefill_tokens))
             out = {"weight_bytes_per_step": engine.weight_bytes_per_step()}
             if not args.only_decode:
@@ -299,7 +355,8 @@ def design_run(args, bracket=None):
             del engine, runs
             torch.cuda.empty_cache()
         print(f"[bench] {size}: {json.dumps(record[size])}", file=sys.stderr, flush=True)
-    print(json.dumps({"metric": "design_throughput", "design": args.design, "beside": "qwen2", "dtype": args.dtype,
+    print(json.dumps({"metric": "design_throughput", "design": args.design,
+                      "beside": "vivevik, qwen2" if args.design == "ninisun" else "qwen2", "dtype": args.dtype,
                       "data": "synthetic", "unit": "tokens/s", "prefill_tokens": args.prefill_tokens,
                       "sizes": record}))
 
@@ -810,10 +867,10 @@ def main():
                     help="fix a choice of the kernels for the whole run, to compare variants: a keyword of "
                          "engine.ops.debug.force, values separated by ':' (attention_splits=64:8, "
                          "attention_merge_kernel=64, gemm_tile=129)")
-    ap.add_argument("--design", choices=["vivevik", "ruvalorn", "minodra"], default=None,
+    ap.add_argument("--design", choices=["vivevik", "ruvalorn", "minodra", "ninisun"], default=None,
                     help="throughput of another design beside the Qwen2 decoder of equal size")
     ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default=None, help="--design: one size only")
-    ap.add_argument("--only-model", choices=["vivevik", "ruvalorn", "minodra", "qwen2"], default=None, help="--design: one of the two models only")
+    ap.add_argument("--only-model", choices=["vivevik", "ruvalorn", "minodra", "ninisun", "qwen2"], default=None, help="--design: one of the two models only")
     ap.add_argument("--only-decode", action="store_true", help="--design: decode at --batch only, no prefill")
     ap.add_argument("--side", choices=["7b", "32b", "f32", "peaks"], help=argparse.SUPPRESS)
     args = ap.parse_args()

@@ -294,17 +294,31 @@ extern "C" int llmlab_gla_output(const float* parts, int rows, int n_heads, int 
 // with w_t (decay) and a_t (removal rate) in (0, 1) per head and key channel.  State [D, E]
 // per head, float32, one slot per request; everything here is float32.
 //
-// delta_gates: w = exp(-decay_scale * sigmoid(w0 + W2 tanh(low))) from the low-rank projection
-// `low` (rank numbers a row), a = sigmoid(a_in + a_bias).
+// delta_gates, one block a row: w = exp(-decay_scale * sigmoid(w0 + W2 tanh(low))) from the
+// low-rank projection `low` (rank numbers a row), a = sigmoid(a_in + a_bias), and what every
+// column of the state needs of the row's key: the unit key u and the removal a * u.
+constexpr int GATES_MAX_HEADS = 1024;
 __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restrict__ proj, int ld, int off_low, int rank,
-                                                          int off_a, const float* __restrict__ w2,
+                                                          int off_a, int off_k, const float* __restrict__ w2,
                                                           const float* __restrict__ w0, const float* __restrict__ a_bias,
-                                                          float decay_scale, float* __restrict__ decay,
-                                                          float* __restrict__ rate, int channels) {
-  extern __shared__ float s_low[];       // tanh of the row's low-rank numbers
-  const int r = blockIdx.x;
+                                                          float decay_scale, float key_eps, float* __restrict__ decay,
+                                                          float* __restrict__ unit, float* __restrict__ removal,
+                                                          int n_heads, int D) {
+  extern __shared__ float s_low[];       // tanh of the row's low-rank numbers, then 1 / |k| of every head
+  float* s_inv = s_low + rank;
+  const int r = blockIdx.x, channels = n_heads * D;
   const float* t = proj + (size_t)r * ld;
   for (int j = threadIdx.x; j < rank; j += blockDim.x) s_low[j] = tanhf(t[off_low + j]);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  for (int h = wave; h < n_heads; h += waves) {          // a wave a head
+    float k2 = 0.f;
+    for (int d = lane; d < D; d += 64) {
+      const float k = t[off_k + h * D + d];
+      k2 = fmaf(k, k, k2);
+    }
+    k2 = wave_sum(k2);
+    if (lane == 0) s_inv[h] = 1.0f / sqrtf(k2 + key_eps);
+  }
   __syncthreads();
   for (int c = threadIdx.x; c < channels; c += blockDim.x) {
     float z = w0 ? w0[c] : 0.f;
@@ -312,106 +326,337 @@ __global__ __launch_bounds__(256) void delta_gates_kernel(const float* __restric
     for (int j = 0; j < rank; ++j) z = fmaf(w[j], s_low[j], z);
     decay[(size_t)r * channels + c] = expf(-decay_scale / (1.0f + expf(-z)));
     const float za = t[off_a + c] + (a_bias ? a_bias[c] : 0.f);
-    rate[(size_t)r * channels + c] = 1.0f / (1.0f + expf(-za));
+    const float u = t[off_k + c] * s_inv[c / D];
+    unit[(size_t)r * channels + c] = u;
+    removal[(size_t)r * channels + c] = u / (1.0f + expf(-za));
   }
 }
 
-extern "C" int llmlab_delta_gates(const float* proj, int ld, int rows, int off_low, int rank, int off_a, const float* w2,
-                                  const float* w0, const float* a_bias, float decay_scale, float* decay, float* rate,
-                                  int channels, hipStream_t stream) {
-  LLMLAB_REQUIRE(rows >= 0 && rank > 0 && rank <= 8192 && channels > 0 && off_low >= 0 && off_a >= 0 &&
-                 ld >= off_low + rank && ld >= off_a + channels,
-                 "delta_gates: bad sizes rows=%d rank=%d channels=%d ld=%d", rows, rank, channels, ld);
+extern "C" int llmlab_delta_gates(const float* proj, int ld, int rows, int off_low, int rank, int off_a, int off_k,
+                                  const float* w2, const float* w0, const float* a_bias, float decay_scale,
+                                  float key_eps, float* decay, float* unit, float* removal, int n_heads, int D,
+                                  hipStream_t stream) {
+  const int channels = n_heads * D;
+  LLMLAB_REQUIRE(rows >= 0 && rank > 0 && rank <= 8192 && n_heads > 0 && n_heads <= GATES_MAX_HEADS && D > 0 &&
+                 off_low >= 0 && off_a >= 0 && off_k >= 0 && ld >= off_low + rank && ld >= off_a + channels &&
+                 ld >= off_k + channels,
+                 "delta_gates: bad sizes rows=%d rank=%d heads=%d D=%d ld=%d", rows, rank, n_heads, D, ld);
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(delta_gates_kernel, dim3(rows), dim3(256), rank * sizeof(float), stream, proj, ld, off_low, rank,
-                     off_a, w2, w0, a_bias, decay_scale, decay, rate, channels);
+  hipLaunchKernelGGL(delta_gates_kernel, dim3(rows), dim3(256), (rank + n_heads) * sizeof(float), stream, proj, ld,
+                     off_low, rank, off_a, off_k, w2, w0, a_bias, decay_scale, key_eps, decay, unit, removal, n_heads, D);
   LLMLAB_LAUNCH_CHECK("delta_gates");
   return 0;
 }
 
-// delta_scan: thread e of block (request, head) keeps column e of the head's state (DK >= D
-// numbers) in registers and walks the request's rows of the step in order; the row's key,
-// receptance, decay and rate are the same for every thread of the block (uniform loads), its
-// value is one number a thread.  No thread talks to another, so a token costs no barrier.
-// Rows [row_begin, row_end) of the request: the state comes from `s_in` and goes to `s_out`
-// (both [D, E] of this head; s_in null: zero).
-template <int DK>
-__device__ __forceinline__ void delta_walk(const float* __restrict__ proj, int ld, int off_r, int off_k, int off_v,
-                                           const float* __restrict__ decay, const float* __restrict__ rate, int n_heads,
-                                           int h, int D, int E, float key_eps, int row_begin, int row_end,
-                                           const float* __restrict__ s_in, float* __restrict__ s_out,
-                                           float* __restrict__ out, int e) {
-  float S[DK];
+// delta_scan.  A quad of lanes keeps ONE column of a head's state in registers, a quarter of its
+// DK >= D numbers each (the two sums over a column meet across the quad), and walks rows in order; the row's decay, unit key, removal, key and receptance are the same for
+// every column: the block brings them into LDS a group of rows ahead (two buffers take turns, one
+// barrier and one wait for memory a group), its value is one number a thread.  Per row and column: the dot product of the unit
+// key with the column, the update, the dot product with the receptance.
+//
+// WHOLE: a block takes all the rows that a request brings to the step, for one head and 64
+// columns: state from the request's slot and back.  Decode steps and short portions.
+//
+// Long portions are cut into chunks that run side by side, in three passes.  The recurrence is
+// linear in the state, S_end = T S_start + L, with T (D x D) the product of the chunk's
+// transitions diag(w) - (a * u) u^T and L the state the chunk builds from zero.  A column of T is
+// what the recurrence without values makes of a unit vector, so:
+//   LOCAL  per chunk: the E columns of L from zero and the D columns of T from the identity, no outputs;
+//   carry  per request, chunk after chunk: S_start[c + 1] = T_c S_start[c] + L_c; the slot at the end;
+//   FINISH per chunk: the rows again from S_start[c], now with outputs.
+enum { DELTA_WHOLE = 0, DELTA_LOCAL = 1, DELTA_FINISH = 2 };
+
+struct DeltaArgs {
+  const float* proj; int ld, off_r, off_k, off_v;
+  const float* decay; const float* unit; const float* removal;      // [rows, heads * D]
+  int n_heads, D, E;
+  float* state; const int* q_start; const int* req_rows; float* out;      // out [rows, heads, E]
+  int n_reqs, chunk; float* chunk_state; float* chunk_trans;      // [chunks, heads, D, E] and [chunks, heads, D, D]
+};
+
+__device__ __forceinline__ bool delta_find_chunk(const DeltaArgs& a, int index, int& first, int& last) {
+  int before = 0;
+  for (int b = 0; b < a.n_reqs; ++b) {
+    const int lo = a.q_start[b], hi = a.q_start[b + 1];
+    const int n = (hi - lo + a.chunk - 1) / a.chunk;
+    if (index < before + n) {
+      first = lo + (index - before) * a.chunk;
+      last = first + a.chunk < hi ? first + a.chunk : hi;
+      return true;
+    }
+    before += n;
+  }
+  return false;
+}
+
+// the sum of a number over the four lanes of a quad (lanes 4 n .. 4 n + 3), in every one of them
+__device__ __forceinline__ float quad_sum(float x) {
+  x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));      // lanes 1, 0, 3, 2
+  x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x4E, 0xF, 0xF, true));      // lanes 2, 3, 0, 1
+  return x;
+}
+
+template <int DK, int MODE>
+__global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs a) {
+  constexpr int VECS = MODE == DELTA_LOCAL ? 4 : 5;      // decay, unit key, removal, key (, receptance)
+  constexpr int DQ = DK / 4;                              // rows of a column that one lane of its quad keeps
+  constexpr int PER = (VECS * DK + 255) / 256;            // numbers of a row that a thread brings
+  constexpr int G = DK <= 64 ? 8 : (DK <= 128 ? 4 : 2);   // rows that travel together (one wait for memory per G rows)
+  __shared__ __attribute__((aligned(16))) float tok[2][G][VECS][DK];
+  const int h = blockIdx.y, D = a.D, E = a.E;
+  const int q = threadIdx.x & 3, d0 = q * DQ;
+  const int col = blockIdx.z * 64 + (int)(threadIdx.x >> 2);
+  const int cols = MODE == DELTA_LOCAL ? E + D : E;
+  int first, last;
+  if (MODE == DELTA_WHOLE) {
+    first = a.q_start[blockIdx.x];
+    last = a.q_start[blockIdx.x + 1];
+  } else if (!delta_find_chunk(a, blockIdx.x, first, last)) {
+    return;
+  }
+  const bool live = col < cols;
+  const bool is_value = col < E;                          // (LOCAL: the others are columns of the transition)
+  const int e = is_value ? col : E - 1;
+  float S[DQ];
+  const float* s_in = MODE == DELTA_WHOLE ? a.state + ((size_t)a.req_rows[blockIdx.x] * a.n_heads + h) * D * E
+                      : MODE == DELTA_FINISH ? a.chunk_state + ((size_t)blockIdx.x * a.n_heads + h) * D * E : nullptr;
 #pragma unroll
-  for (int d = 0; d < DK; ++d) S[d] = (s_in && d < D && e < E) ? s_in[(size_t)d * E + e] : 0.f;
-  const int ec = e < E ? e : E - 1;
-  for (int t = row_begin; t < row_end; ++t) {
-    const float* row = proj + (size_t)t * ld;
-    const float* kk = row + off_k + h * D;
-    const float* rr = row + off_r + h * D;
-    const float* ww = decay + ((size_t)t * n_heads + h) * D;
-    const float* aa = rate + ((size_t)t * n_heads + h) * D;
-    const float v = row[off_v + h * E + ec];
-    float k2 = 0.f;
+  for (int i = 0; i < DQ; ++i) {
+    const int d = d0 + i;
+    if (MODE == DELTA_LOCAL) S[i] = (live && !is_value && d == col - E) ? 1.f : 0.f;
+    else S[i] = (live && d < D) ? s_in[(size_t)d * E + e] : 0.f;
+  }
+  // the numbers of a row that this thread brings: number i of vector i / D, for i = tid, tid + 256, ...
+  const int total = VECS * D;
+  float pre[G][PER], v_pre[G], v_now[G];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int d = 0; d < DK; ++d)
-      if (d < D) k2 = fmaf(kk[d], kk[d], k2);
-    const float inv = 1.0f / sqrtf(k2 + key_eps);
-    float dot = 0.f;
+    for (int g = 0; g < G; ++g) {
+      if (g > 0 && t0 + g >= last) break;                          // (a decode step brings one row)
+      const int t = t0 + g;
+      const float* row = a.proj + (size_t)t * a.ld;
+      const size_t at = ((size_t)t * a.n_heads + h) * D;
+      v_pre[g] = is_value ? row[a.off_v + h * E + e] : 0.f;
 #pragma unroll
-    for (int d = 0; d < DK; ++d)
-      if (d < D) dot = fmaf(kk[d] * inv, S[d], dot);
-    float o = 0.f;
-#pragma unroll
-    for (int d = 0; d < DK; ++d)
-      if (d < D) {
-        const float k = kk[d];
-        S[d] = fmaf(ww[d], S[d], fmaf(-(aa[d] * (k * inv)), dot, k * v));
-        o = fmaf(S[d], rr[d], o);
+      for (int n = 0; n < PER; ++n) {
+        const int i = threadIdx.x + n * 256;
+        float x = 0.f;
+        if (i < total) {
+          const int vec = i / D, d = i - vec * D;
+          x = vec == 0 ? a.decay[at + d] : vec == 1 ? a.unit[at + d] : vec == 2 ? a.removal[at + d]
+              : vec == 3 ? row[a.off_k + h * D + d] : row[a.off_r + h * D + d];
+        }
+        pre[g][n] = x;
       }
-    if (e < E) out[((size_t)t * n_heads + h) * E + e] = o;
-  }
-  if (e < E) {
+    }
+  };
+  auto stash = [&](int buf, int t0) {
 #pragma unroll
-    for (int d = 0; d < DK; ++d)
-      if (d < D) s_out[(size_t)d * E + e] = S[d];
+    for (int g = 0; g < G; ++g) {
+      if (g > 0 && t0 + g >= last) break;
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        const int i = threadIdx.x + n * 256;
+        if (i < total) {
+          const int vec = i / D, d = i - vec * D;
+          tok[buf][g][vec][d] = pre[g][n];
+        }
+      }
+    }
+  };
+  // (vectors shorter than DK: the rest stays zero, so the sums over DK numbers need no bound)
+  if (D < DK)
+    for (int i = threadIdx.x; i < 2 * G * VECS * DK; i += 256) (&tok[0][0][0][0])[i] = 0.f;
+  __syncthreads();
+  if (first < last) {
+    fetch(first);
+    stash(0, first);
   }
+  __syncthreads();
+  for (int t0 = first, buf = 0; t0 < last; t0 += G, buf ^= 1) {
+#pragma unroll
+    for (int g = 0; g < G; ++g) v_now[g] = v_pre[g];
+    const bool more = t0 + G < last;
+    if (more) fetch(t0 + G);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const int t = t0 + g;
+      if (t < last) {
+        const float v = v_now[g];
+        const float* w_ = &tok[buf][g][0][d0];
+        const float* u_ = &tok[buf][g][1][d0];
+        const float* au_ = &tok[buf][g][2][d0];
+        const float* k_ = &tok[buf][g][3][d0];
+        // (sums side by side, so that no sum waits for the one before it)
+        float dots[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < DQ; ++i) dots[i & 3] = fmaf(u_[i], S[i], dots[i & 3]);
+        const float dot = quad_sum((dots[0] + dots[1]) + (dots[2] + dots[3]));
+        float os[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < DQ; ++i) {
+          S[i] = fmaf(w_[i], S[i], fmaf(-au_[i], dot, k_[i] * v));
+          if (MODE != DELTA_LOCAL) os[i & 3] = fmaf(S[i], tok[buf][g][VECS - 1][d0 + i], os[i & 3]);
+        }
+        if (MODE != DELTA_LOCAL) {
+          const float o = quad_sum((os[0] + os[1]) + (os[2] + os[3]));
+          if (live && q == 0) a.out[((size_t)t * a.n_heads + h) * E + e] = o;
+        }
+      }
+    }
+    if (more) stash(buf ^ 1, t0 + G);
+    __syncthreads();
+  }
+  if (MODE == DELTA_FINISH || !live) return;
+  float* dst;
+  size_t stride;
+  if (MODE == DELTA_WHOLE) {
+    dst = a.state + ((size_t)a.req_rows[blockIdx.x] * a.n_heads + h) * D * E + e;
+    stride = E;
+  } else if (is_value) {
+    dst = a.chunk_state + ((size_t)blockIdx.x * a.n_heads + h) * D * E + e;
+    stride = E;
+  } else {
+    dst = a.chunk_trans + ((size_t)blockIdx.x * a.n_heads + h) * D * D + (col - E);
+    stride = D;
+  }
+#pragma unroll
+  for (int i = 0; i < DQ; ++i)
+    if (d0 + i < D) dst[(size_t)(d0 + i) * stride] = S[i];
 }
 
+// carry: block (request, head, slab of 16 columns), CARRY_GROUPS waves; wave g computes the rows
+// g, g + CARRY_GROUPS, ... of T_c S + L_c for the slab's columns: a column a quad of lanes, each lane
+// a quarter of the sum over the old rows.  The slab of the state and the chunk's transition lie in
+// LDS (a wave brings its own rows of the transition, the next chunk's while this chunk's sums are
+// taken).  chunk_state[c] <- the state before chunk c.
+constexpr int CARRY_GROUPS = 8, CARRY_COLS = 16;
 template <int DK>
-__global__ __launch_bounds__(256) void delta_scan_kernel(const float* __restrict__ proj, int ld, int off_r, int off_k,
-                                                         int off_v, const float* __restrict__ decay,
-                                                         const float* __restrict__ rate, int n_heads, int D, int E,
-                                                         float key_eps, float* __restrict__ state,
-                                                         const int* __restrict__ q_start, const int* __restrict__ req_rows,
-                                                         float* __restrict__ out) {
-  const int b = blockIdx.x, h = blockIdx.y;
-  const int e = blockIdx.z * blockDim.x + threadIdx.x;
-  float* st = state + ((size_t)req_rows[b] * n_heads + h) * D * E;
-  delta_walk<DK>(proj, ld, off_r, off_k, off_v, decay, rate, n_heads, h, D, E, key_eps, q_start[b], q_start[b + 1], st, st,
-                 out, e);
+__global__ __launch_bounds__(64 * CARRY_GROUPS) void delta_carry_kernel(DeltaArgs a) {
+  constexpr int ROWS = (DK + CARRY_GROUPS - 1) / CARRY_GROUPS, M = (DK + 63) / 64, DQ = DK / 4;
+  __shared__ __attribute__((aligned(16))) float s_tr[ROWS * CARRY_GROUPS][DK + 4];
+  __shared__ float s_col[DK][CARRY_COLS + 1];
+  const int b = blockIdx.x, h = blockIdx.y, D = a.D, E = a.E;
+  const int lane = threadIdx.x & 63, g = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int q = lane & 3, c16 = lane >> 2, j0 = q * DQ;
+  const int e = blockIdx.z * CARRY_COLS + c16;
+  const bool live = e < E;
+  const int ec = live ? e : E - 1;
+  int before = 0;
+  for (int r = 0; r < b; ++r) before += (a.q_start[r + 1] - a.q_start[r] + a.chunk - 1) / a.chunk;
+  const int n = (a.q_start[b + 1] - a.q_start[b] + a.chunk - 1) / a.chunk;
+  float* slot = a.state + ((size_t)a.req_rows[b] * a.n_heads + h) * D * E;
+  for (int i = threadIdx.x; i < DK * CARRY_COLS; i += blockDim.x) {
+    const int d = i / CARRY_COLS, c = i % CARRY_COLS;
+    const int ee = blockIdx.z * CARRY_COLS + c;
+    s_col[d][c] = (d < D && ee < E) ? slot[(size_t)d * E + ee] : 0.f;
+  }
+  // this wave's rows of a chunk's transition (64 entries of a row a register) and of its built state
+  float tr[ROWS][M], built[ROWS];
+  auto fetch = [&](int c) {
+    const float* lp = a.chunk_state + ((size_t)c * a.n_heads + h) * D * E;
+    const float* tp = a.chunk_trans + ((size_t)c * a.n_heads + h) * D * D;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+      const int d = g + CARRY_GROUPS * i;
+      built[i] = d < D ? lp[(size_t)d * E + ec] : 0.f;
+#pragma unroll
+      for (int m = 0; m < M; ++m) tr[i][m] = (d < D && 64 * m + lane < D) ? tp[(size_t)d * D + 64 * m + lane] : 0.f;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        if (64 * m + lane < DK) s_tr[g + CARRY_GROUPS * i][64 * m + lane] = tr[i][m];
+  };
+  if (n > 0) {
+    fetch(before);
+    stash();
+  }
+  __syncthreads();
+  for (int c = before; c < before + n; ++c) {
+    float acc[ROWS];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) acc[i] = q == 0 ? built[i] : 0.f;
+    if (c + 1 < before + n) fetch(c + 1);                          // (on its way while the sums are taken)
+    float* l = a.chunk_state + ((size_t)c * a.n_heads + h) * D * E;
+#pragma unroll
+    for (int jj = 0; jj < DQ; ++jj) {
+      const float x = s_col[j0 + jj][c16];
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) acc[i] = fmaf(s_tr[g + CARRY_GROUPS * i][j0 + jj], x, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) acc[i] = quad_sum(acc[i]);
+    if (live && q == 0) {                                          // the state before this chunk, in the chunk's place
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) {
+        const int d = g + CARRY_GROUPS * i;
+        if (d < D) l[(size_t)d * E + e] = s_col[d][c16];
+      }
+    }
+    __syncthreads();                                               // (every wave has read the old columns and the transition)
+    if (q == 0) {
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) {
+        const int d = g + CARRY_GROUPS * i;
+        if (d < DK) s_col[d][c16] = acc[i];
+      }
+    }
+    if (c + 1 < before + n) stash();
+    __syncthreads();
+  }
+  if (live && q == 0)
+    for (int d = g; d < D; d += CARRY_GROUPS) slot[(size_t)d * E + e] = s_col[d][c16];
 }
 
+// proj [rows, ld] float32 holds r at off_r (heads * D), k at off_k, v at off_v (heads * E); decay,
+// unit and removal [rows, heads * D] (delta_gates); state [slots, heads, D, E]; out [rows, heads, E].
+// chunk > 0: the three-pass form over chunks of so many rows; chunk_state then holds max_chunks *
+// heads * D * E floats and chunk_trans max_chunks * heads * D * D, max_chunks >= rows / chunk + n_reqs.
 extern "C" int llmlab_delta_scan(const float* proj, int ld, int off_r, int off_k, int off_v, const float* decay,
-                                 const float* rate, int n_heads, int D, int E, float key_eps, float* state,
-                                 const int* q_start, const int* req_rows, int n_reqs, float* out, int rows,
-                                 hipStream_t stream) {
-  LLMLAB_REQUIRE(rows >= 0 && n_reqs >= 0 && n_heads > 0 && n_heads <= 65535 && D > 0 && D <= 256 && E > 0 && E <= 16384,
+                                 const float* unit, const float* removal, int n_heads, int D, int E, float* state,
+                                 const int* q_start, const int* req_rows, int n_reqs, float* out, int rows, int chunk,
+                                 float* chunk_state, float* chunk_trans, int max_chunks, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && n_reqs >= 0 && n_reqs <= 65535 && n_heads > 0 && n_heads <= 65535 && D > 0 && D <= 256 &&
+                 E > 0 && E <= 16384,
                  "delta_scan: bad sizes rows=%d requests=%d heads=%d D=%d E=%d (keys up to 256 wide)", rows, n_reqs,
                  n_heads, D, E);
   LLMLAB_REQUIRE(off_r >= 0 && off_k >= 0 && off_v >= 0 && ld >= off_r + n_heads * D && ld >= off_k + n_heads * D &&
                  ld >= off_v + n_heads * E, "delta_scan: rows of %d numbers do not hold the projections", ld);
   if (rows == 0 || n_reqs == 0) return 0;
-  const int threads = E <= 64 ? 64 : (E <= 128 ? 128 : 256);
-  dim3 grid(n_reqs, n_heads, (E + threads - 1) / threads), block(threads);
-#define LLMLAB_DELTA(DKV)                                                                                             \
-  hipLaunchKernelGGL(delta_scan_kernel<DKV>, grid, block, 0, stream, proj, ld, off_r, off_k, off_v, decay, rate, n_heads, \
-                     D, E, key_eps, state, q_start, req_rows, out)
-  if (D <= 16) LLMLAB_DELTA(16);
-  else if (D <= 32) LLMLAB_DELTA(32);
-  else if (D <= 64) LLMLAB_DELTA(64);
-  else if (D <= 128) LLMLAB_DELTA(128);
-  else LLMLAB_DELTA(256);
+  DeltaArgs a{proj, ld, off_r, off_k, off_v, decay, unit, removal, n_heads, D, E, state, q_start, req_rows, out,
+              n_reqs, chunk, chunk_state, chunk_trans};
+#define LLMLAB_DELTA(DKV, MODE, GRIDX, COLS) \
+  hipLaunchKernelGGL((delta_scan_kernel<DKV, MODE>), dim3(GRIDX, n_heads, ((COLS) + 63) / 64), dim3(256), 0, stream, a)
+#define LLMLAB_DELTA_ANY(MODE, GRIDX, COLS)                   \
+  do {                                                        \
+    if (D <= 16) LLMLAB_DELTA(16, MODE, GRIDX, COLS);         \
+    else if (D <= 32) LLMLAB_DELTA(32, MODE, GRIDX, COLS);    \
+    else if (D <= 64) LLMLAB_DELTA(64, MODE, GRIDX, COLS);    \
+    else if (D <= 128) LLMLAB_DELTA(128, MODE, GRIDX, COLS);  \
+    else LLMLAB_DELTA(256, MODE, GRIDX, COLS);                \
+  } while (0)
+  LLMLAB_REQUIRE((E + 63) / 64 <= 65535 && (E + D + 63) / 64 <= 65535, "delta_scan: too many columns");
+  if (chunk <= 0) {
+    LLMLAB_DELTA_ANY(DELTA_WHOLE, n_reqs, E);
+  } else {
+    const int chunks = rows / chunk + n_reqs;
+    LLMLAB_REQUIRE(chunk_state && chunk_trans && max_chunks >= chunks,
+                   "delta_scan: %d rows of %d requests in chunks of %d need room for %d chunks, got %d", rows, n_reqs,
+                   chunk, chunks, max_chunks);
+    LLMLAB_REQUIRE(D <= 128, "delta_scan: chunks take states of up to 128 key channels, got %d", D);
+    LLMLAB_DELTA_ANY(DELTA_LOCAL, chunks, E + D);
+    const dim3 cgrid(n_reqs, n_heads, (E + CARRY_COLS - 1) / CARRY_COLS), cblock(64 * CARRY_GROUPS);
+    if (D <= 16) hipLaunchKernelGGL(delta_carry_kernel<16>, cgrid, cblock, 0, stream, a);
+    else if (D <= 32) hipLaunchKernelGGL(delta_carry_kernel<32>, cgrid, cblock, 0, stream, a);
+    else if (D <= 64) hipLaunchKernelGGL(delta_carry_kernel<64>, cgrid, cblock, 0, stream, a);
+    else hipLaunchKernelGGL(delta_carry_kernel<128>, cgrid, cblock, 0, stream, a);
+    LLMLAB_DELTA_ANY(DELTA_FINISH, chunks, E);
+  }
+#undef LLMLAB_DELTA_ANY
 #undef LLMLAB_DELTA
   LLMLAB_LAUNCH_CHECK("delta_scan");
   return 0;

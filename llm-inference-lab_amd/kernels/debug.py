@@ -71,6 +71,8 @@ class DispatchRules:
     scan_min_chunk: int = 16
     scan_max_chunk: int = 64
     scan_blocks_per_cu: int = 1
+    # the delta rule's scan joins its chunks with a dense transition each: longer chunks, fewer joins
+    delta_scan_max_chunk: int = 128
     # Windowed attention with a sink: a request that brings at least this many rows to a step is
     # served by the matrix-core kernel (tiles of 16 rows of one request), the others row by row
     # by the plain kernel.  64 decoding requests in tiles of 16 rows of 16 requests: 14.3 ms a

@@ -1116,12 +1116,13 @@ class HipOps:
                 lib.llmlab_gla_output.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr,
                                                   _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
                 lib.llmlab_gla_output.restype = _c_int
-                lib.llmlab_delta_gates.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
-                                                   _c_ptr, _c_float, _c_ptr, _c_ptr, _c_int, _c_ptr]
+                lib.llmlab_delta_gates.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                                                   _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                                                   _c_ptr]
                 lib.llmlab_delta_gates.restype = _c_int
-                lib.llmlab_delta_scan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
-                                                  _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int,
-                                                  _c_ptr]
+                lib.llmlab_delta_scan.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                                                  _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int,
+                                                  _c_ptr, _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_delta_scan.restype = _c_int
             elif kind == "routed_experts":
                 lib.llmlab_moe_select.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
@@ -1594,15 +1595,21 @@ class HipOps:
                    float(eps), self._ptr(proj), proj.stride(0), int(off_gate), self._ptr(out), _dt(out),
                    int(parts.shape[2]), per_head, self.OUTPUT_GATES[gate], self._stream(), lib=lib)
 
-    def delta_gates(self, proj, off_low, rank, off_rate, w2, w0, rate_bias, decay_scale, decay, rate) -> None:
-        """``decay[r, c] = exp(-decay_scale * sigmoid(w0[c] + w2[c] . tanh(proj[r, off_low : off_low + rank])))``
-        and ``rate[r, c] = sigmoid(proj[r, off_rate + c] + rate_bias[c])``, all float32."""
+    def delta_gates(self, proj, off_low, rank, off_rate, off_k, w2, w0, rate_bias, decay_scale, key_eps, num_heads,
+                    key_dim, decay, unit, removal) -> None:
+        """What the delta rule's scan needs of every row, all float32 ``[rows, heads * key_dim]``:
+        ``decay[r, c] = exp(-decay_scale * sigmoid(w0[c] + w2[c] . tanh(proj[r, off_low : off_low + rank])))``,
+        the unit key ``unit = k / sqrt(|k|^2 + key_eps)`` head by head (``k`` at column ``off_k`` of
+        ``proj``), and ``removal = sigmoid(proj[r, off_rate + c] + rate_bias[c]) * unit``."""
         lib = self._mixer_lib("linear_attention")
-        for t, name in ((proj, "projections"), (w2, "decay weight"), (decay, "decays"), (rate, "rates")):
+        for t, name in ((proj, "projections"), (w2, "decay weight"), (decay, "decays"), (unit, "unit keys"),
+                        (removal, "removals")):
             self._need(t, name, torch.float32)
         rows, channels = decay.shape
-        if (proj.shape[0] != rows or tuple(rate.shape) != (rows, channels) or tuple(w2.shape) != (channels, rank)
-                or off_low < 0 or off_low + rank > proj.shape[1] or off_rate < 0 or off_rate + channels > proj.shape[1]):
+        if (proj.shape[0] != rows or tuple(unit.shape) != (rows, channels) or tuple(removal.shape) != (rows, channels)
+                or channels != num_heads * key_dim or tuple(w2.shape) != (channels, rank)
+                or min(off_low, off_rate, off_k) < 0 or off_low + rank > proj.shape[1]
+                or max(off_rate, off_k) + channels > proj.shape[1]):
             raise ValueError("delta_gates: the operands do not fit each other")
         for t, name in ((w0, "decay bias"), (rate_bias, "rate bias")):
             if t is not None:
@@ -1610,31 +1617,64 @@ class HipOps:
                 if t.numel() != channels:
                     raise ValueError(f"delta_gates: one {name} per channel")
         self._call(lib.llmlab_delta_gates, self._ptr(proj), proj.stride(0), rows, int(off_low), int(rank), int(off_rate),
-                   self._ptr(w2), self._ptr(w0), self._ptr(rate_bias), float(decay_scale), self._ptr(decay),
-                   self._ptr(rate), channels, self._stream(), lib=lib)
+                   int(off_k), self._ptr(w2), self._ptr(w0), self._ptr(rate_bias), float(decay_scale), float(key_eps),
+                   self._ptr(decay), self._ptr(unit), self._ptr(removal), int(num_heads), int(key_dim), self._stream(),
+                   lib=lib)
 
-    def delta_scan(self, proj, off_r, off_k, off_v, decay, rate, num_heads, key_dim, value_dim, key_eps, state, q_start,
-                   req_rows, n_reqs, out) -> None:
-        """The recurrence ``S = diag(decay_t) S - (rate_t * u_t)(u_t^T S) + k_t v_t^T; o_t = S^T r_t`` with
-        ``u_t = k_t / sqrt(|k_t|^2 + key_eps)`` over the rows ``q_start[b] .. q_start[b + 1]`` of each of the
-        step's ``n_reqs`` requests, on the float32 state ``state[req_rows[b]]`` ``[heads, key_dim,
-        value_dim]``, which is left updated; ``out [rows, heads, 1, value_dim]`` float32."""
+    DELTA_CHUNK_MAX_KEYS = 128      # wider states walk their rows in one run (a column no longer fits the registers)
+
+    def delta_scan_chunk(self, rows: int, longest: int, num_heads: int, key_dim: int, value_dim: int) -> int:
+        """Into chunks of how many rows the delta rule's scan cuts a step whose longest request brings
+        ``longest`` rows (0: every request's rows in one run).  Chunks run side by side at the price of
+        walking the rows twice, once more for the chunk's transition, and of joining the chunks one
+        after the other; so short runs stay whole, and the chunks are as long as still gives every
+        compute unit a block."""
+        if longest < 2 * self.rules.scan_min_chunk or key_dim > self.DELTA_CHUNK_MAX_KEYS:
+            return 0
+        per_chunk = num_heads * ((value_dim + key_dim + 255) // 256)
+        chunk = self.rules.delta_scan_max_chunk
+        while chunk > self.rules.scan_min_chunk and (rows // chunk) * per_chunk < self.rules.scan_blocks_per_cu * self.num_cus:
+            chunk //= 2
+        return chunk
+
+    def delta_scan(self, proj, off_r, off_k, off_v, decay, unit, removal, num_heads, key_dim, value_dim, state, q_start,
+                   req_rows, n_reqs, out, chunk=0, chunk_state=None, chunk_trans=None) -> None:
+        """The recurrence ``S = diag(decay_t) S - removal_t (unit_t^T S) + k_t v_t^T; o_t = S^T r_t`` over the
+        rows ``q_start[b] .. q_start[b + 1]`` of each of the step's ``n_reqs`` requests, on the float32 state
+        ``state[req_rows[b]]`` ``[heads, key_dim, value_dim]``, which is left updated; ``out [rows, heads, 1,
+        value_dim]`` float32.  ``chunk > 0``: every request's rows in chunks of so many that run side by
+        side, joined afterwards (``chunk_state [chunks, heads, key_dim, value_dim]`` and ``chunk_trans
+        [chunks, heads, key_dim, key_dim]`` float32 scratch, ``chunks >= rows // chunk + n_reqs``)."""
         lib = self._mixer_lib("linear_attention")
-        for t, name in ((proj, "projections"), (decay, "decays"), (rate, "rates"), (state, "recurrent state"),
-                        (out, "outputs")):
+        if key_dim > self.DELTA_CHUNK_MAX_KEYS:        # (the chunks' kernels take narrower states only)
+            chunk = 0
+        for t, name in ((proj, "projections"), (decay, "decays"), (unit, "unit keys"), (removal, "removals"),
+                        (state, "recurrent state"), (out, "outputs")):
             self._need(t, name, torch.float32)
         self._need(q_start, "request row starts", torch.int32)
         self._need(req_rows, "state slots", torch.int32)
         rows = proj.shape[0]
-        if (tuple(decay.shape) != (rows, num_heads * key_dim) or tuple(rate.shape) != tuple(decay.shape)
-                or out.numel() != rows * num_heads * value_dim
+        if (tuple(decay.shape) != (rows, num_heads * key_dim) or tuple(unit.shape) != tuple(decay.shape)
+                or tuple(removal.shape) != tuple(decay.shape) or out.numel() != rows * num_heads * value_dim
                 or tuple(state.shape[1:]) != (num_heads, key_dim, value_dim)
                 or q_start.numel() < n_reqs + 1 or req_rows.numel() < n_reqs or min(off_r, off_k, off_v) < 0
                 or max(off_r + num_heads * key_dim, off_k + num_heads * key_dim, off_v + num_heads * value_dim) > proj.shape[1]):
             raise ValueError("delta_scan: the operands do not fit each other")
+        max_chunks = 0
+        if chunk:
+            self._need(chunk_state, "chunk states", torch.float32)
+            self._need(chunk_trans, "chunk transitions", torch.float32)
+            max_chunks = chunk_state.shape[0]
+            if (tuple(chunk_state.shape[1:]) != (num_heads, key_dim, value_dim)
+                    or tuple(chunk_trans.shape) != (max_chunks, num_heads, key_dim, key_dim)
+                    or max_chunks < rows // chunk + n_reqs):
+                raise ValueError(f"delta_scan: the scratch of the chunks does not fit {rows} rows of {n_reqs} requests "
+                                 f"in chunks of {chunk}")
         self._call(lib.llmlab_delta_scan, self._ptr(proj), proj.stride(0), int(off_r), int(off_k), int(off_v),
-                   self._ptr(decay), self._ptr(rate), num_heads, key_dim, value_dim, float(key_eps), self._ptr(state),
-                   self._ptr(q_start), self._ptr(req_rows), int(n_reqs), self._ptr(out), rows, self._stream(), lib=lib)
+                   self._ptr(decay), self._ptr(unit), self._ptr(removal), num_heads, key_dim, value_dim, self._ptr(state),
+                   self._ptr(q_start), self._ptr(req_rows), int(n_reqs), self._ptr(out), rows, int(chunk),
+                   self._ptr(chunk_state) if chunk else None, self._ptr(chunk_trans) if chunk else None, max_chunks,
+                   self._stream(), lib=lib)
 
     # --------------------------------------------------------------- sampling
     # ------------------------------ the stream around sublayers; the latent form of attention

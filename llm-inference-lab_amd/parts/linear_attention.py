@@ -247,6 +247,10 @@ class DeltaRuleAttention(Mixer):
         self.b_rate = tensors[t["rate_bias"]].float().contiguous()
         self.norm_weight = tensors[t["out_norm"]].float().contiguous()
 
+    def _min_chunk(self) -> int:
+        rules = getattr(self.ops, "rules", None)
+        return int(getattr(rules, "scan_min_chunk", 16))
+
     def state_spec(self):
         return {"s": ((self.num_heads, self.key_dim, self.value_dim), torch.float32)}
 
@@ -255,18 +259,28 @@ class DeltaRuleAttention(Mixer):
         proj = ctx.scratch("delta_rule.proj", (rows, self.in_size), torch.float32)
         ops.linear_logits(h, self.w_in, proj)
         decay = ctx.scratch("delta_rule.decay", (rows, self.qk_size), torch.float32)
-        rate = ctx.scratch("delta_rule.rate", (rows, self.qk_size), torch.float32)
-        ops.delta_gates(proj, o["decay_down"], self.decay_rank, o["rate_weight"], self.w_decay, self.b_decay,
-                        self.b_rate, self.decay_scale, decay, rate)
+        unit = ctx.scratch("delta_rule.unit", (rows, self.qk_size), torch.float32)
+        removal = ctx.scratch("delta_rule.removal", (rows, self.qk_size), torch.float32)
+        ops.delta_gates(proj, o["decay_down"], self.decay_rank, o["rate_weight"], o["k_weight"], self.w_decay,
+                        self.b_decay, self.b_rate, self.decay_scale, self.key_eps, self.num_heads, self.key_dim, decay,
+                        unit, removal)
         outs = ctx.scratch("delta_rule.outputs", (rows, self.num_heads, 1, self.value_dim), torch.float32)
         state = entry.state["s"]
+        # room for the chunks of a long portion: at most rows / (smallest chunk) + requests
+        most = rows // max(1, self._min_chunk()) + ctx.max_reqs
+        chunk_state = ctx.scratch("delta_rule.chunk_state", (most, self.num_heads, self.key_dim, self.value_dim),
+                                  torch.float32)
+        chunk_trans = ctx.scratch("delta_rule.chunk_trans", (most, self.num_heads, self.key_dim, self.key_dim),
+                                  torch.float32)
 
         def scan():
-            # (how many requests the step has is read when the launch is made, also when it is made
-            # again from a kept sequence of calls)
-            ops.delta_scan(proj, o["r_weight"], o["k_weight"], o["v_weight"], decay, rate, self.num_heads,
-                           self.key_dim, self.value_dim, self.key_eps, state, ctx.all_q_start, ctx.all_req_rows,
-                           ctx.n_reqs, outs)
+            # (how many requests the step has and how long the longest portion is are read when the
+            # launch is made, also when it is made again from a kept sequence of calls)
+            pick = getattr(ops, "delta_scan_chunk", None)
+            chunk = (pick(rows, ctx.max_q_len, self.num_heads, self.key_dim, self.value_dim) if pick is not None else 0)
+            ops.delta_scan(proj, o["r_weight"], o["k_weight"], o["v_weight"], decay, unit, removal, self.num_heads,
+                           self.key_dim, self.value_dim, state, ctx.all_q_start, ctx.all_req_rows, ctx.n_reqs, outs,
+                           chunk, chunk_state if chunk else None, chunk_trans if chunk else None)
         live = getattr(ops, "live", None)
         if live is not None:
             live(scan)

@@ -356,20 +356,31 @@ class EmuOps:
     def check_delta_rule_sizes(self, num_heads, key_dim, value_dim):
         pass
 
-    def delta_gates(self, proj, off_low, rank, off_rate, w2, w0, rate_bias, decay_scale, decay, rate):
+    def delta_gates(self, proj, off_low, rank, off_rate, off_k, w2, w0, rate_bias, decay_scale, key_eps, num_heads,
+                    key_dim, decay, unit, removal):
         self._count("delta_gates")
+        channels = num_heads * key_dim
         z = torch.tanh(proj[:, off_low:off_low + rank].float()) @ w2.float().t()
         if w0 is not None:
             z = z + w0.float()
         decay.copy_(torch.exp(-decay_scale * torch.sigmoid(z)))
-        za = proj[:, off_rate:off_rate + decay.shape[1]].float()
+        za = proj[:, off_rate:off_rate + channels].float()
         if rate_bias is not None:
             za = za + rate_bias.float()
-        rate.copy_(torch.sigmoid(za))
+        k = proj[:, off_k:off_k + channels].float().view(-1, num_heads, key_dim)
+        u = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + key_eps)).reshape(-1, channels)
+        unit.copy_(u)
+        removal.copy_(torch.sigmoid(za) * u)
 
-    def delta_scan(self, proj, off_r, off_k, off_v, decay, rate, num_heads, key_dim, value_dim, key_eps, state, q_start,
-                   req_rows, n_reqs, out):
+    def delta_scan_chunk(self, rows, longest, num_heads, key_dim, value_dim):
+        return 16 if longest >= 32 else 0
+
+    def delta_scan(self, proj, off_r, off_k, off_v, decay, unit, removal, num_heads, key_dim, value_dim, state, q_start,
+                   req_rows, n_reqs, out, chunk=0, chunk_state=None, chunk_trans=None):
+        """(``chunk``: how the kernel spreads the work; the recurrence is the same.)"""
         self._count("delta_scan")
+        if chunk:
+            assert chunk_state.shape[0] >= proj.shape[0] // chunk + n_reqs and chunk_trans.shape[0] == chunk_state.shape[0]
         H, D, E = num_heads, key_dim, value_dim
         o = out.view(-1, H, E)
         for b in range(n_reqs):
@@ -378,9 +389,8 @@ class EmuOps:
                 r = proj[t, off_r:off_r + H * D].view(H, D)
                 k = proj[t, off_k:off_k + H * D].view(H, D)
                 v = proj[t, off_v:off_v + H * E].view(H, E)
-                u = k / torch.sqrt((k * k).sum(-1, keepdim=True) + key_eps)
-                dot = torch.einsum("hd,hde->he", u, st)
-                new = (decay[t].view(H, D, 1) * st - (rate[t].view(H, D) * u).unsqueeze(-1) * dot.unsqueeze(-2)
+                dot = torch.einsum("hd,hde->he", unit[t].view(H, D), st)
+                new = (decay[t].view(H, D, 1) * st - removal[t].view(H, D, 1) * dot.unsqueeze(-2)
                        + k.unsqueeze(-1) * v.unsqueeze(-2))
                 st.copy_(new)
                 o[t] = torch.einsum("hde,hd->he", st, r)

@@ -245,31 +245,42 @@ def test_softmax_without_a_sink_at_the_window_s_edges(backend, dtype, H_, G, D, 
 
 # ------------------------------------------------------------------ the delta rule
 @pytest.mark.parametrize("backend", BACKENDS)
-def test_decays_and_removal_rates(backend):
+def test_decays_removal_rates_and_unit_keys(backend):
     ops = ops_of(backend)
-    rows, rank, channels = 11, 5, 52
-    proj = randn(rows, 3 + rank + channels, seed=1, scale=3.0).to(ops.device)
+    rows, rank, heads, D = 11, 5, 4, 13
+    channels = heads * D
+    proj = randn(rows, 3 + rank + 2 * channels, seed=1, scale=3.0)
+    proj[3, 3 + rank + channels:3 + rank + channels + D] = 0.0            # a key of length zero: the eps keeps it finite
+    proj = proj.to(ops.device)
     w2 = randn(channels, rank, seed=2, scale=2.0).to(ops.device)
     w0 = randn(channels, seed=3, scale=10.0).to(ops.device)                 # both ends of the sigmoid
     ab = randn(channels, seed=4, scale=5.0).to(ops.device)
-    decay, rate = torch.empty(rows, channels, device=ops.device), torch.empty(rows, channels, device=ops.device)
-    ops.delta_gates(proj, 3, rank, 3 + rank, w2, w0, ab, math.exp(-0.5), decay, rate)
+    decay, unit, removal = (torch.empty(rows, channels, device=ops.device) for _ in range(3))
+    ops.delta_gates(proj, 3, rank, 3 + rank, 3 + rank + channels, w2, w0, ab, math.exp(-0.5), 1e-6, heads, D, decay, unit,
+                    removal)
     p = proj.cpu().to(F64)
     z = torch.tanh(p[:, 3:3 + rank]) @ w2.cpu().to(F64).T + w0.cpu().to(F64)
     close(decay, torch.exp(-math.exp(-0.5) * torch.sigmoid(z)), torch.float32, "decays", f32=3e-6)
-    close(rate, torch.sigmoid(p[:, 3 + rank:] + ab.cpu().to(F64)), torch.float32, "rates", f32=3e-6)
+    k = p[:, 3 + rank + channels:].view(rows, heads, D)
+    u = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)).reshape(rows, channels)
+    close(unit, u, torch.float32, "unit keys", f32=3e-6)
+    close(removal, torch.sigmoid(p[:, 3 + rank:3 + rank + channels] + ab.cpu().to(F64)) * u, torch.float32, "removals", f32=3e-6)
     assert float(decay.min()) >= math.exp(-math.exp(-0.5)) - 1e-6 and float(decay.max()) <= 1.0
+    assert torch.isfinite(unit).all()
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("heads,D,E", [(2, 16, 16), (3, 24, 24), (1, 40, 40), (2, 64, 64), (1, 128, 128), (2, 8, 72), (1, 200, 16)])
-def test_delta_rule_scan_in_portions_with_states_in_slots(backend, heads, D, E):
+@pytest.mark.parametrize("chunk", [0, 16, 32])
+@pytest.mark.parametrize("heads,D,E", [(2, 16, 16), (3, 24, 24), (1, 40, 40), (2, 64, 64), (1, 128, 128), (2, 8, 72), (1, 200, 16),
+                                       (1, 32, 300)])
+def test_delta_rule_scan_in_portions_with_states_in_slots(backend, heads, D, E, chunk):
     """Three requests of unequal length in one call, then their next portions (down to one token) in
     a second one from the states the first left in scattered slots, against the plain recurrence over
-    the whole sequences; a slot that is zeroed starts anew."""
+    the whole sequences; whole runs and chunks that run side by side (chunks that end inside a
+    request's rows, requests shorter than a chunk)."""
     ops = ops_of(backend)
     dev = ops.device
-    lengths, first = [37, 5, 64], [20, 4, 2]
+    lengths, first = [137, 5, 64], [90, 4, 2]
     ld = 3 * heads * D + heads * E + 7
     off_r, off_k, off_v = 5, 5 + heads * D, 5 + 2 * heads * D
     state = torch.zeros(6, heads, D, E, device=dev)
@@ -280,26 +291,30 @@ def test_delta_rule_scan_in_portions_with_states_in_slots(backend, heads, D, E):
         proj = randn(n, ld, seed=10 + b)
         decay = torch.exp(-0.6 * torch.rand(n, heads * D, generator=torch.Generator().manual_seed(20 + b)))
         rate = torch.rand(n, heads * D, generator=torch.Generator().manual_seed(30 + b))
-        data.append((proj, decay, rate))
         r, k = proj[:, off_r:off_r + heads * D].view(n, heads, D), proj[:, off_k:off_k + heads * D].view(n, heads, D)
         v = proj[:, off_v:off_v + heads * E].view(n, heads, E)
+        unit = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)).reshape(n, -1)
+        data.append((proj, decay, unit, rate * unit))
         wants.append(_plain_delta(r.to(F64), k.to(F64), v.to(F64), decay.view(n, heads, D).to(F64),
                                   rate.view(n, heads, D).to(F64)))
     for part in (0, 1):
         spans = [(0, first[b]) if part == 0 else (first[b], lengths[b]) for b in range(3)]
-        proj = torch.cat([data[b][0][lo:hi] for b, (lo, hi) in enumerate(spans)]).to(dev)
-        decay = torch.cat([data[b][1][lo:hi] for b, (lo, hi) in enumerate(spans)]).to(dev)
-        rate = torch.cat([data[b][2][lo:hi] for b, (lo, hi) in enumerate(spans)]).to(dev)
+        proj, decay, unit, removal = (torch.cat([data[b][i][lo:hi] for b, (lo, hi) in enumerate(spans)]).to(dev)
+                                      for i in range(4))
         starts = [0]
         for lo, hi in spans:
             starts.append(starts[-1] + hi - lo)
-        out = torch.full((proj.shape[0], heads, 1, E), float("nan"), device=dev)
-        ops.delta_scan(proj, off_r, off_k, off_v, decay, rate, heads, D, E, 1e-6, state,
-                       torch.tensor(starts, dtype=torch.int32, device=dev), slots, 3, out)
+        rows = proj.shape[0]
+        out = torch.full((rows, heads, 1, E), float("nan"), device=dev)
+        most = rows // chunk + 3 if chunk else 0
+        ops.delta_scan(proj, off_r, off_k, off_v, decay, unit, removal, heads, D, E, state,
+                       torch.tensor(starts, dtype=torch.int32, device=dev), slots, 3, out, chunk,
+                       torch.full((most, heads, D, E), float("nan"), device=dev) if chunk else None,
+                       torch.full((most, heads, D, D), float("nan"), device=dev) if chunk else None)
         for b, (lo, hi) in enumerate(spans):
-            close(out[starts[b]:starts[b + 1], :, 0], wants[b][0][lo:hi], torch.float32, f"request {b}, part {part}", f32=2e-5)
+            close(out[starts[b]:starts[b + 1], :, 0], wants[b][0][lo:hi], torch.float32, f"request {b}, part {part}", f32=3e-5)
     for b in range(3):
-        close(state[int(slots[b])], wants[b][1], torch.float32, f"state of request {b}", f32=2e-5)
+        close(state[int(slots[b])], wants[b][1], torch.float32, f"state of request {b}", f32=3e-5)
     assert float((state[4] - 9.0).abs().max()) == 0.0
 
 
