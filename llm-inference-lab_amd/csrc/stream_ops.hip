@@ -4,7 +4,8 @@
 //   norm_conv       the RMS norm of the stream's rows and that convolution over them in one launch
 //   gated_add       x += y * sigmoid(gate + bias)
 //   softcap         x = cap * tanh(x / cap)
-//   rmsnorm_add     x += y / sqrt(mean(y^2) + eps) * w   (a norm on a sublayer's result, before the sum)
+//   rmsnorm_add     x += y / sqrt(mean(y^2) + eps) * w   (a norm on a sublayer's result, before the sum;
+//                   the norm that reads the stream next may run in the same launch)
 //   scaled_sum      out = a * y1 + b * y2
 // What a request's earlier steps left (its last token, the last inputs of a convolution) lives in
 // per-request slots; a step's rows of one request are adjacent.
@@ -409,9 +410,13 @@ extern "C" int llmlab_gated_add(float* x, const float* y, int pieces, size_t pie
 // pieces, in the pieces' order).  All float32.  A thread keeps up to NORM_ADD_KEEP of the row's numbers
 // in registers between the two passes; wider rows are read again.
 constexpr int NORM_ADD_KEEP = 8;
+// NEXT: the norm that reads the stream next runs in the same launch on the row's new numbers:
+// next_out[r, c] = T(x[r, c] / sqrt(mean(x[r]^2) + next_eps) * next_w[c]).
+template <typename T, bool NEXT>
 __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ x, const float* __restrict__ y, int pieces,
                                                           size_t piece_stride, const float* __restrict__ w, float eps,
-                                                          int width) {
+                                                          int width, const float* __restrict__ next_w, float next_eps,
+                                                          T* __restrict__ next_out) {
   __shared__ float red[17];
   const size_t row = (size_t)blockIdx.x * width;
   float keep[NORM_ADD_KEEP];
@@ -432,20 +437,48 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ x,
     ss = fmaf(v, v, ss);
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)width + eps);
+  float ss2 = 0.f;
 #pragma unroll
   for (int n = 0; n < NORM_ADD_KEEP; ++n) {
     const int c = threadIdx.x + 256 * n;
-    if (c < width) x[row + c] += keep[n] * inv * w[c];
+    if (c < width) {
+      keep[n] = x[row + c] + keep[n] * inv * w[c];
+      x[row + c] = keep[n];
+      ss2 = fmaf(keep[n], keep[n], ss2);
+    }
   }
-  for (int c = threadIdx.x + 256 * NORM_ADD_KEEP; c < width; c += 256) x[row + c] += value(c) * inv * w[c];
+  for (int c = threadIdx.x + 256 * NORM_ADD_KEEP; c < width; c += 256) {
+    const float v = x[row + c] + value(c) * inv * w[c];
+    x[row + c] = v;
+    ss2 = fmaf(v, v, ss2);
+  }
+  if (!NEXT) return;
+  const float inv2 = 1.0f / sqrtf(block_sum(ss2, red) / (float)width + next_eps);
+#pragma unroll
+  for (int n = 0; n < NORM_ADD_KEEP; ++n) {
+    const int c = threadIdx.x + 256 * n;
+    if (c < width) next_out[row + c] = from_float<T>(keep[n] * inv2 * next_w[c]);
+  }
+  for (int c = threadIdx.x + 256 * NORM_ADD_KEEP; c < width; c += 256)      // (what this thread itself has just written)
+    next_out[row + c] = from_float<T>(x[row + c] * inv2 * next_w[c]);
 }
 
 extern "C" int llmlab_rmsnorm_add(float* x, const float* y, int pieces, size_t piece_stride, const float* w, float eps,
-                                  int rows, int width, hipStream_t stream) {
+                                  int rows, int width, const float* next_w, float next_eps, void* next_out,
+                                  int next_dtype, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && width > 0 && pieces >= 1 && x && y && w, "rmsnorm_add: bad arguments rows=%d width=%d pieces=%d",
                  rows, width, pieces);
+  LLMLAB_REQUIRE((next_w == nullptr) == (next_out == nullptr), "rmsnorm_add: the next norm needs its weight and its output");
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(rows), dim3(256), 0, stream, x, y, pieces, piece_stride, w, eps, width);
+  if (!next_out)
+    hipLaunchKernelGGL((rmsnorm_add_kernel<float, false>), dim3(rows), dim3(256), 0, stream, x, y, pieces, piece_stride, w,
+                       eps, width, nullptr, 0.f, nullptr);
+  else if (next_dtype == DT_BF16)
+    hipLaunchKernelGGL((rmsnorm_add_kernel<bf16_t, true>), dim3(rows), dim3(256), 0, stream, x, y, pieces, piece_stride, w,
+                       eps, width, next_w, next_eps, (bf16_t*)next_out);
+  else
+    hipLaunchKernelGGL((rmsnorm_add_kernel<float, true>), dim3(rows), dim3(256), 0, stream, x, y, pieces, piece_stride, w,
+                       eps, width, next_w, next_eps, (float*)next_out);
   LLMLAB_LAUNCH_CHECK("rmsnorm_add");
   return 0;
 }

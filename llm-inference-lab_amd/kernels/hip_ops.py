@@ -1099,7 +1099,7 @@ class HipOps:
                 lib.llmlab_softcap.argtypes = [_c_ptr, _c_float, _c_size, _c_ptr]
                 lib.llmlab_softcap.restype = _c_int
                 lib.llmlab_rmsnorm_add.argtypes = [_c_ptr, _c_ptr, _c_int, _c_size, _c_ptr, _c_float, _c_int, _c_int,
-                                                   _c_ptr]
+                                                   _c_ptr, _c_float, _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_rmsnorm_add.restype = _c_int
                 lib.llmlab_scaled_sum.argtypes = [_c_ptr, _c_ptr, _c_float, _c_ptr, _c_float, _c_size, _c_ptr]
                 lib.llmlab_scaled_sum.restype = _c_int
@@ -1810,10 +1810,12 @@ class HipOps:
         self._call(lib.llmlab_gated_add, self._ptr(x), self._ptr(y), pieces, piece_stride, self._ptr(gate), cols,
                    self._ptr(bias), rows, width, self._stream(), lib=lib)
 
-    def rmsnorm_add(self, y, weight, eps: float, x) -> None:
+    def rmsnorm_add(self, y, weight, eps: float, x, next_norm=None) -> None:
         """``x += y / sqrt(mean(y^2) + eps) * weight`` row by row, all float32: the norm of a sublayer's
         result on its way into the stream.  ``y [rows, width]``, or a product left in pieces
-        (``PendingSums``), which are summed on the way."""
+        (``PendingSums``), which are summed on the way.  ``next_norm = (weight, eps, out)``: the RMS norm
+        that reads the stream next, in the same launch: ``out = norm(x)`` of the new rows (float32
+        weight, ``out`` in a kernel dtype)."""
         lib = self._mixer_lib("stream_ops")
         self._need(x, "stream", torch.float32)
         self._need(weight, "norm weight", torch.float32)
@@ -1831,8 +1833,17 @@ class HipOps:
             parts, pieces, stride = y, 1, 0
         if weight.numel() != width:
             raise ValueError("rmsnorm_add: one weight per column")
+        next_w = next_out = None
+        next_eps = 0.0
+        if next_norm is not None:
+            next_w, next_eps, next_out = next_norm
+            self._need(next_w, "next norm's weight", torch.float32)
+            self._need(next_out, "next norm's output")
+            if next_w.numel() != width or tuple(next_out.shape) != (rows, width):
+                raise ValueError("rmsnorm_add: the next norm's weight and output have the stream's shape")
         self._call(lib.llmlab_rmsnorm_add, self._ptr(x), self._ptr(parts), int(pieces), int(stride), self._ptr(weight),
-                   float(eps), rows, width, self._stream(), lib=lib)
+                   float(eps), rows, width, self._ptr(next_w), float(next_eps), self._ptr(next_out),
+                   _dt(next_out) if next_out is not None else 0, self._stream(), lib=lib)
 
     def scaled_sum(self, out, y1, a: float, y2, b: float) -> None:
         """``out = a * y1 + b * y2``, float32 tensors of one shape."""

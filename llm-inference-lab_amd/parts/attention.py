@@ -8,7 +8,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..weights.loader import TensorSpec, MATRIX, VECTOR, INIT_NORM
-from .base import Mixer, KVCacheSpec, CacheSpec, PageTensor, NormedInput, PendingSums
+from .base import Mixer, KVCacheSpec, CacheSpec, PageTensor, NormedInput, PendingSums, project_normed
 from .registry import register_part, build_part
 
 
@@ -324,6 +324,7 @@ class WindowedSinkAttention(Mixer):
     Pages: keys ``[kv_heads, P, key_dim]``, values ``[kv_heads, P, value_dim]``."""
 
     writes_output = True
+    takes_normed_input = True      # (few rows: the norm in front of the mixer runs inside its first product)
     WEIGHTS = ("softmax", "sigmoid")
     VALUE_MIX = (None, "first", "mix")
 
@@ -453,7 +454,7 @@ class WindowedSinkAttention(Mixer):
                              "and one that has them writes its own")
         group = ctx.group(entry.group)
         proj = ctx.scratch("windowed_attention.proj", (rows, self.in_size), torch.float32)
-        ops.linear_logits(h, self.w_in, proj)
+        project_normed(ops, h, self.w_in, proj, self.dtype, self.hidden_size)
         q = ctx.scratch("windowed_attention.q", (rows, self.q_size), self.dtype)
         gate = None
         if self.rotates:
@@ -496,8 +497,6 @@ class WindowedSinkAttention(Mixer):
         ops.linear_logits(mixed, self.w_o, out)
 
     def forward(self, h, residual, ctx, entry):
-        if isinstance(h, NormedInput):
-            h = h.tensor()
         y = ctx.scratch("windowed_attention.sum", (1,) + tuple(residual.shape), torch.float32)
         self.forward_into(h, y[0], ctx, entry)
         self.ops.add_pending(residual, PendingSums(y, 1))

@@ -213,6 +213,21 @@ class NormedInput:
         return self._tensor
 
 
+def project_normed(ops, h, weight, out, dtype, hidden_size: int) -> None:
+    """``out = h W^T`` in float32 for a mixer's first product, where ``h`` is a tensor of normed
+    activations or a ``NormedInput``: few rows of an RMS norm go through the kernel that norms the
+    rows as it stages them, anything else through the norm and the product."""
+    if isinstance(h, NormedInput):
+        fuse = (ops.can_fuse(out.shape[0], dtype, hidden_size, out.shape[1])
+                and not ops.pieces_too_large_to_read_per_block(getattr(h.ctx, "pending", None)))
+        rms = h.rms() if fuse else None
+        if rms is not None:
+            ops.fused_norm_logits(rms[0], rms[1], rms[2], rms[3], weight, out)
+            return
+        h = h.tensor()
+    ops.linear_logits(h, weight, out)
+
+
 class PositionEncoding(Part):
     def rotary_table(self) -> Optional[torch.Tensor]:
         """``inv_freq [rotary_dim/2]`` float32 if this is a split-half rotation

@@ -174,6 +174,7 @@ class SandwichNormBlock(Block):
         self.feed_forward = build_part("feed_forward", feed_forward) if feed_forward is not None else None
         self.post_norm2 = build_part("norm", post_norm2) if post_norm2 is not None else None
         self.post = [None, None]       # (weight with the layer scale folded in, eps) of each half
+        self.next_weight, self.next_eps = None, 0.0      # the feed-forward's norm, if it is an RMS norm
 
     def parts(self):
         return [p for p in (self.norm1, self.mixer, self.post_norm1, self.norm2, self.feed_forward, self.post_norm2)
@@ -206,6 +207,9 @@ class SandwichNormBlock(Block):
             if role in self.tensor_names:
                 weight = weight * tensors[self.tensor_names[role]].float()
             self.post[i] = (weight.contiguous(), float(params[1]))
+        params = self.norm2.rms_params() if self.norm2 is not None and hasattr(self.norm2, "rms_params") else None
+        if params is not None:
+            self.next_weight, self.next_eps = params[0].float().contiguous(), float(params[1])
 
     def kernel_libraries(self):
         return [("stream_ops", None)] + super().kernel_libraries()
@@ -216,11 +220,13 @@ class SandwichNormBlock(Block):
             self.ops.add_pending(residual, pending)
             ctx.pending = None
 
-    def _half(self, i, norm, part, residual, ctx, *view):
+    def _half(self, i, h, part, residual, ctx, next_norm, *view):
+        """One sublayer: ``h`` is its input (a tensor, or a ``NormedInput`` for a part that may fold
+        the norm into its first product); ``next_norm``: the norm that reads the stream next, to run
+        in the launch of the sum."""
         ops, rows = self.ops, residual.shape[0]
-        self._fold(residual, ctx)
-        h = ctx.scratch("block.normed", (rows, self.hidden_size), self.dtype)
-        norm.forward(residual, h)
+        if isinstance(h, NormedInput) and not part.takes_normed_input:
+            h = h.tensor()
         y = ctx.scratch("block.sublayer_out", (rows, self.hidden_size), torch.float32)
         if part.writes_output:
             part.forward_into(h, y, ctx, *view)
@@ -233,12 +239,24 @@ class SandwichNormBlock(Block):
             part.forward(h, y, ctx, *view)
             self._fold(y, ctx)
         weight, eps = self.post[i]
-        ops.rmsnorm_add(y, weight, eps, residual)
+        if next_norm is not None:
+            ops.rmsnorm_add(y, weight, eps, residual, next_norm)
+        else:
+            ops.rmsnorm_add(y, weight, eps, residual)
 
     def forward(self, residual, ctx, entry):
-        self._half(0, self.norm1, self.mixer, residual, ctx, entry)
-        if self.feed_forward is not None:
-            self._half(1, self.norm2, self.feed_forward, residual, ctx)
+        self._fold(residual, ctx)
+        h = NormedInput(self.norm1, residual, ctx, "block.normed", self.dtype)
+        if self.feed_forward is None:
+            self._half(0, h, self.mixer, residual, ctx, None, entry)
+            return
+        # the feed-forward's norm runs in the launch that sums the mixer's result into the stream
+        h2 = ctx.scratch("block.normed2", (residual.shape[0], self.hidden_size), self.dtype)
+        self._half(0, h, self.mixer, residual, ctx, (self.next_weight, self.next_eps, h2) if self.next_weight is not None else None,
+                   entry)
+        if self.next_weight is None:
+            self.norm2.forward(residual, h2)
+        self._half(1, h2, self.feed_forward, residual, ctx, None)
 
     def weight_bytes(self):
         own = sum(w.numel() * w.element_size() for w, _ in (p for p in self.post if p is not None))

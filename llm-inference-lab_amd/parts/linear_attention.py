@@ -6,7 +6,7 @@ from typing import Dict, Optional
 import torch
 
 from ..weights.loader import TensorSpec, MATRIX, VECTOR, INIT_NORM
-from .base import Mixer, NormedInput, PendingSums
+from .base import Mixer, NormedInput, PendingSums, project_normed
 from .registry import register_part
 
 
@@ -177,6 +177,7 @@ class DeltaRuleAttention(Mixer):
     decay_up, decay_bias, out_norm, o_weight``."""
 
     writes_output = True
+    takes_normed_input = True
     keeps_launches = True
     DEFAULT_DECAY_SCALE = 0.6065306597126334      # exp(-1/2)
 
@@ -257,7 +258,7 @@ class DeltaRuleAttention(Mixer):
     def forward_into(self, h, out, ctx, entry):
         ops, rows, o = self.ops, h.shape[0], self.offsets
         proj = ctx.scratch("delta_rule.proj", (rows, self.in_size), torch.float32)
-        ops.linear_logits(h, self.w_in, proj)
+        project_normed(ops, h, self.w_in, proj, self.dtype, self.hidden_size)
         decay = ctx.scratch("delta_rule.decay", (rows, self.qk_size), torch.float32)
         unit = ctx.scratch("delta_rule.unit", (rows, self.qk_size), torch.float32)
         removal = ctx.scratch("delta_rule.removal", (rows, self.qk_size), torch.float32)
@@ -292,8 +293,6 @@ class DeltaRuleAttention(Mixer):
         ops.linear_logits(mixed, self.w_o, out)
 
     def forward(self, h, residual, ctx, entry):
-        if isinstance(h, NormedInput):
-            h = h.tensor()
         y = ctx.scratch("delta_rule.sum", (1,) + tuple(residual.shape), torch.float32)
         self.forward_into(h, y[0], ctx, entry)
         self.ops.add_pending(residual, PendingSums(y, 1))

@@ -17,6 +17,7 @@ class ParallelMixers(Mixer):
     under the names they give it, which must differ."""
 
     writes_output = True
+    takes_normed_input = True      # (each of the two takes it as it can; the norm itself runs at most once)
 
     def __init__(self, left: PartSpec, right: PartSpec, left_scale: float = 1.0, right_scale: float = 1.0,
                  tensors: Optional[Dict[str, str]] = None):
@@ -62,6 +63,8 @@ class ParallelMixers(Mixer):
         return [("stream_ops", None)] + [lib for m in self.members() for lib in m.kernel_libraries()]
 
     def _result(self, mixer, name, h, shape, ctx, entry):
+        if isinstance(h, NormedInput) and not mixer.takes_normed_input:
+            h = h.tensor()
         y = ctx.scratch(name, shape, torch.float32)
         if mixer.writes_output:
             mixer.forward_into(h, y, ctx, entry)
@@ -81,8 +84,6 @@ class ParallelMixers(Mixer):
         self.ops.scaled_sum(out, y1, self.left_scale, y2, self.right_scale)
 
     def forward(self, h, residual, ctx, entry):
-        if isinstance(h, NormedInput):
-            h = h.tensor()
         y = ctx.scratch("parallel.sum", (1,) + tuple(residual.shape), torch.float32)
         self.forward_into(h, y[0], ctx, entry)
         self.ops.add_pending(residual, PendingSums(y, 1))

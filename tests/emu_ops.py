@@ -395,10 +395,13 @@ class EmuOps:
                 st.copy_(new)
                 o[t] = torch.einsum("hde,hd->he", st, r)
 
-    def rmsnorm_add(self, y, weight, eps, x):
+    def rmsnorm_add(self, y, weight, eps, x, next_norm=None):
         self._count("rmsnorm_add")
         v = self._owed(y) if isinstance(y, PendingSums) else y.float()
         x.add_(v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight.float())
+        if next_norm is not None:
+            w, e, out = next_norm
+            out.copy_((x / torch.sqrt((x * x).mean(-1, keepdim=True) + e) * w.float()).to(out.dtype))
 
     def scaled_sum(self, out, y1, a, y2, b):
         self._count("scaled_sum")

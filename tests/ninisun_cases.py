@@ -18,7 +18,9 @@ def rot(dims, base, scaling=None):
 
 
 def attention(heads, kv_heads, dim, vdim, scale, rotation, size=None, keep_first=0, v_mix=False, ff=None):
-    mixer = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, rot=rotation, v_mix=v_mix)
+    mixer = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, v_mix=v_mix)
+    if rotation is not None:
+        mixer["rot"] = rotation
     if size is not None:
         mixer["mask"] = dict(size=size, keep_first=keep_first)
     return dict(type="attention", mixer=mixer, mlp=None if ff is None else dict(kind="dense", ff=ff))
@@ -26,9 +28,12 @@ def attention(heads, kv_heads, dim, vdim, scale, rotation, size=None, keep_first
 
 def parallel(left, right, left_scale, right_scale, ff=None):
     heads, kv_heads, dim, vdim, scale, rotation = left
+    side = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale)
+    if rotation is not None:
+        side["rot"] = rotation
     return dict(type="parallel",
-                mixer=dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, rot=rotation),
-                           right=dict(heads=right[0], dim=right[1]), left_scale=left_scale, right_scale=right_scale),
+                mixer=dict(left=side, right=dict(heads=right[0], dim=right[1]), left_scale=left_scale,
+                           right_scale=right_scale),
                 mlp=None if ff is None else dict(kind="dense", ff=ff))
 
 

@@ -112,8 +112,8 @@ def windowed_mixer(h, p, m, v_first=None):
     q = (h @ p["q"].T).view(T, H, D)
     k = (h @ p["k"].T).view(T, G, D)
     v = (h @ p["v"].T).view(T, G, E)
-    pos = range(T)
-    q, k = rotate_pairs(q, pos, m["rot"]), rotate_pairs(k, pos, m["rot"])
+    if m.get("rot"):
+        q, k = rotate_pairs(q, range(T), m["rot"]), rotate_pairs(k, range(T), m["rot"])
     if v_first is not None:
         lam = p["vmix"]
         v = (1.0 - lam) * v + lam * v_first
@@ -129,8 +129,8 @@ def gated_sigmoid_mixer(h, p, m):
     q = (h @ p["q"].T + p["q.b"]).view(T, H, D)
     k = (h @ p["k"].T + p["k.b"]).view(T, G, D)
     v = (h @ p["v"].T + p["v.b"]).view(T, G, E)
-    pos = range(T)
-    q, k = rotate_pairs(q, pos, m["rot"]), rotate_pairs(k, pos, m["rot"])
+    if m.get("rot"):
+        q, k = rotate_pairs(q, range(T), m["rot"]), rotate_pairs(k, range(T), m["rot"])
     o = sigmoid_attention(q, k, v, m["scale"], p["pb"])
     o = o * torch.sigmoid(h @ p["g"].T).unsqueeze(-1)
     return o.reshape(T, H * E) @ p["o"].T

@@ -33,6 +33,15 @@ def test_norm_of_a_result_into_the_stream(backend, hidden):
     want = x2.cpu().to(F64) + P.rms_norm(pieces[:3].cpu().to(F64).sum(0), w.cpu().to(F64), 1e-3)
     ops.rmsnorm_add(PendingSums(pieces, 3), w, 1e-3, x2)
     close(x2, want, torch.float32, "stream += norm(sum of pieces)", f32=3e-6)
+    # the norm that reads the stream next, in the same launch
+    for dtype in DTYPES:
+        x3 = randn(9, hidden, seed=6).to(dev)
+        w_next = (1.0 + randn(hidden, seed=7, scale=0.3)).to(dev)
+        h = torch.full((9, hidden), float("nan"), dtype=dtype, device=dev)
+        want = x3.cpu().to(F64) + P.rms_norm(y.cpu().to(F64), w.cpu().to(F64), 1e-5)
+        ops.rmsnorm_add(y, w, 1e-5, x3, (w_next, 1e-6, h))
+        close(x3, want, torch.float32, "stream += norm(y), with the next norm", f32=3e-6)
+        close(h, P.rms_norm(want, w_next.cpu().to(F64), 1e-6), dtype, "the next norm of the new rows")
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
