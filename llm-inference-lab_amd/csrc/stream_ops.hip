@@ -419,17 +419,21 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ x,
                                                           T* __restrict__ next_out) {
   __shared__ float red[17];
   const size_t row = (size_t)blockIdx.x * width;
-  float keep[NORM_ADD_KEEP];
+  float keep[NORM_ADD_KEEP], xs[NORM_ADD_KEEP], ws[NORM_ADD_KEEP];
   float ss = 0.f;
   auto value = [&](int c) {
     float v = y[row + c];
     for (int s = 1; s < pieces; ++s) v += y[s * piece_stride + row + c];
     return v;
   };
+  // (the stream's numbers and the weights are asked for together with the result's, before the
+  // first sum is reduced: one trip to memory a row)
 #pragma unroll
   for (int n = 0; n < NORM_ADD_KEEP; ++n) {
     const int c = threadIdx.x + 256 * n;
     keep[n] = c < width ? value(c) : 0.f;
+    xs[n] = c < width ? x[row + c] : 0.f;
+    ws[n] = c < width ? w[c] : 0.f;
     ss = fmaf(keep[n], keep[n], ss);
   }
   for (int c = threadIdx.x + 256 * NORM_ADD_KEEP; c < width; c += 256) {
@@ -442,7 +446,7 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ x,
   for (int n = 0; n < NORM_ADD_KEEP; ++n) {
     const int c = threadIdx.x + 256 * n;
     if (c < width) {
-      keep[n] = x[row + c] + keep[n] * inv * w[c];
+      keep[n] = xs[n] + keep[n] * inv * ws[n];
       x[row + c] = keep[n];
       ss2 = fmaf(keep[n], keep[n], ss2);
     }
