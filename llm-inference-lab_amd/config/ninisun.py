@@ -62,11 +62,12 @@ class NinisunRotation:
     def check(self, dim: int, at: str) -> None:
         if self.dims < 0 or self.dims % 2 or self.dims > dim:
             raise ConfigError(f"{at}: rot.dims {self.dims} must be even and at most the head's {dim} channels")
-        if not (math.isfinite(self.base) and self.base > 1.0):
-            raise ConfigError(f"{at}: rot.base must be finite and > 1, got {self.base}")
+        if not (math.isfinite(self.base) and self.base > 0.0):
+            raise ConfigError(f"{at}: rot.base must be finite and > 0, got {self.base}")
         s = self.scaling
-        if s is not None and not (s.factor >= 1.0 and s.original > 0 and s.fast > 0 and s.slow > 0):
-            raise ConfigError(f"{at}: rot.scaling needs factor >= 1 and positive original, fast and slow, got {s}")
+        if s is not None and not (s.factor > 0 and s.original > 0 and s.fast > 0 and s.slow > 0 and self.base != 1.0):
+            raise ConfigError(f"{at}: rot.scaling needs positive factor, original, fast and slow (and a base other "
+                              f"than 1), got {s}")
 
 
 @dataclasses.dataclass(frozen=True)

@@ -80,8 +80,10 @@ def softmax_attention(q, k, v, scale, size=None, keep_first=0, q_positions=None)
     if q_positions is None:
         q_positions = list(range(S - T, S))
     out = torch.zeros(T, H, E, dtype=q.dtype)
+    every = torch.arange(S)
     for t, i in enumerate(q_positions):
-        js = torch.tensor([j for j in range(S) if visible(i, j, size, keep_first)])
+        # (the keys that ``visible`` admits, all at once)
+        js = every[(every <= i) & ((i - every < (size if size is not None else S + 1)) | (every < keep_first))]
         for hd in range(H):
             g = hd // (H // G)
             s = (k[js, g] @ q[t, hd]) * scale

@@ -178,3 +178,21 @@ def test_greedy_generation_through_the_scheduler(backend):
             ids.append(token)
     engine.cache.check()
     assert engine.cache.metrics()["rows_used"] == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_decode_steps_replayed_from_a_graph(dtype):
+    """Decode steps captured into a HIP graph and replayed, with the program's own eager steps
+    (new requests' prompts) between the replays: every token the one an engine without graphs
+    computes.  More requests than rows, so slots are reused between replays."""
+    name = "P"
+    cfg = N.config_of(name)
+    prompts = [N.random_ids(cfg, n, 40 + n) for n in (7, 30, 12, 3)]
+    runs = {}
+    for graph in (False, True):
+        engine = N.make_engine(name, 1, dtype, page_size=16, num_pages=40, max_requests=2, max_batch_tokens=32, graph=graph)
+        runs[graph] = engine.generate(prompts, max_new_tokens=40)
+        if graph:
+            assert engine.metrics()["graphs"]["replays"] > 20
+    assert runs[True] == runs[False]

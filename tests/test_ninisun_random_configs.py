@@ -95,6 +95,50 @@ def test_drawn_configuration(backend, seed):
         assert engine.cache.metrics()["rows_used"] == 0
 
 
+# Two configurations at the sizes of small real models: head sizes that the matrix-core attention
+# kernels take (groups of 4 heads and of 3 share their keys), values twice as wide as keys on the
+# left, states of 64 x 64 and 128 x 128 (scans in chunks), windows that cross the 64-token pages.
+REAL = {
+    "M": dict(architecture="Ninisun", vocab=1000, width=256, norm=dict(eps=1e-6), layers=[
+        N.attention(8, 2, 64, 64, 0.125, N.rot(32, 5e5), size=100, keep_first=4, v_mix=True, ff=512),
+        N.parallel((8, 2, 64, 128, 0.125, N.rot(16, 1e6, (4.0, 256, 32.0, 1.0))), (4, 64), 0.8, 0.9, ff=512),
+        N.attention(8, 2, 64, 64, 0.125, N.rot(32, 5e5), size=100, keep_first=4, v_mix=True, ff=512),
+    ]),
+    "N": dict(architecture="Ninisun", vocab=777, width=384, norm=dict(eps=1e-5), layers=[
+        N.parallel((6, 2, 128, 128, 0.09, N.rot(64, 1e4)), (2, 128), 1.1, 0.6, ff=640),
+        N.attention(6, 6, 32, 96, 0.18, N.rot(32, 1e4, (2.0, 128, 8.0, 0.5)), size=70, keep_first=0, v_mix=True),
+        N.attention(12, 6, 96, 96, 0.1, N.rot(8, 1e6), v_mix=True, ff=200),
+    ]),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(REAL))
+def test_sizes_of_small_real_models(name):
+    cfg = H.lab.NinisunConfig.from_dict(REAL[name])
+    tensors = N.make_tensors(cfg, 3)
+    for t in tensors:                       # (wider rows: products of order one again)
+        if tensors[t].dim() == 2 and t != "embed" and not t.endswith((".w1", ".w2")):
+            tensors[t] = (tensors[t].float() * 0.5).to(torch.bfloat16)
+    seqs = {f"r{i}": N.random_ids(cfg, n, 50 + i) for i, n in enumerate([260, 45, 130, 200])}
+    want = {rid: plain_ninisun.forward(cfg.to_dict(), tensors, ids) for rid, ids in seqs.items()}
+    size = max(1.0, float(torch.cat(list(want.values())).std()))
+    for dtype in ("f32", "bf16"):
+        for cut in (H.steps_prefill_then_decode, lambda s: H.steps_mixed(s, seed=1, max_live=3, budget=192)):
+            engine = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=64, num_pages=20,
+                                  max_requests=3, max_batch_tokens=320, max_seq_len=320)
+            got = H.run_trace(engine, seqs, cut(seqs))
+            diff = torch.cat([got[rid].double() - want[rid] for rid in got])
+            assert not torch.isnan(diff).any()
+            if dtype == "f32":
+                bad = H.first_wrong(got, want, 5e-4 * size)
+                assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+            else:
+                rms = float(diff.pow(2).mean().sqrt())
+                assert rms < 0.06 * size, rms
+            engine.cache.check()
+
+
 def test_configuration_round_trip_and_errors():
     """``to_dict`` gives back what ``from_dict`` read; what cannot be a model of this design is refused
     with the place named."""
