@@ -916,9 +916,9 @@ __global__ __launch_bounds__(64) void sink_window_attention_merge_kernel(MfmaArg
 // Whether the matrix-core kernel takes these sizes at all.
 extern "C" int llmlab_sink_window_attention_has_mfma(int dtype, int D, int E, int page_size) {
   if (g_force_plain || dtype != DT_BF16 || D % 32 != 0 || E % 16 != 0 || page_size % 16 != 0) return 0;
-  // (keys and values up to 128 wide in any combination; wider ones, up to 256, where both are of
-  // one width: the latent form, whose values are its keys)
-  return (D <= 128 && E <= 128) || (D == E && D <= 256);
+  // (keys and values up to 128 wide in any combination; values of 192 and 256 beside keys of 64 to
+  // 128; wider keys, up to 256, where both are of one width: the latent form, whose values are its keys)
+  return (D <= 128 && E <= 128) || (D >= 64 && D <= 128 && (E == 192 || E == 256)) || (D == E && D <= 256);
 }
 
 template <int DC>
@@ -931,6 +931,9 @@ static void launch_mfma(int EBv, int which, dim3 grid, dim3 block, hipStream_t s
     break;
   switch (EBv) {
     LLMLAB_MFMA(1) LLMLAB_MFMA(2) LLMLAB_MFMA(3) LLMLAB_MFMA(4) LLMLAB_MFMA(5) LLMLAB_MFMA(6) LLMLAB_MFMA(7) LLMLAB_MFMA(8)
+  }
+  if constexpr (DC >= 2) {      // (values of 192 and 256 beside keys of 64 to 128)
+    switch (EBv) { LLMLAB_MFMA(12) LLMLAB_MFMA(16) }
   }
 #undef LLMLAB_MFMA
 }

@@ -184,7 +184,8 @@ def _attend(cache, rows_q, H_, positions, row_req, window, keep_first, head_term
 
 
 # sizes with and without matrix-core kernels; groups of 1, 2, 4 and 7 heads per key/value head
-SHAPES = [(4, 2, 16, 24), (4, 2, 32, 16), (8, 2, 96, 64), (3, 1, 64, 48), (14, 2, 64, 64), (2, 2, 24, 200), (8, 2, 96, 192)]
+SHAPES = [(4, 2, 16, 24), (4, 2, 32, 16), (8, 2, 96, 64), (3, 1, 64, 48), (14, 2, 64, 64), (2, 2, 24, 200), (8, 2, 96, 192),
+          (4, 1, 128, 256), (6, 2, 64, 192), (2, 2, 32, 192)]
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -216,7 +217,7 @@ def test_sigmoid_weights_over_prompts_and_decoded_rows(backend, dtype, H_, G, D,
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H_,G,D,E", [(4, 2, 16, 24), (4, 2, 32, 16), (8, 2, 64, 32)])
+@pytest.mark.parametrize("H_,G,D,E", [(4, 2, 16, 24), (4, 2, 32, 16), (8, 2, 64, 32), (8, 2, 96, 192), (2, 1, 128, 256)])
 @pytest.mark.parametrize("window,keep_first", [(24, 3), (16, 0), (5, 9), (40, 6), (300, 2)])
 def test_softmax_without_a_sink_at_the_window_s_edges(backend, dtype, H_, G, D, E, window, keep_first):
     """The plain softmax (no sink) through a window with a kept prefix: a key that would take nearly
