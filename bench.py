@@ -259,12 +259,12 @@ def ninisun_config(size):
     for i in range(layers):
         if i % 3 == 0:
             left = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5,
-                        rot=dict(dims=dim // 2, base=1e6, scaling=dict(factor=4.0, original=1024, fast=32.0, slow=1.0)))
-            mixer = dict(left=left, right=dict(heads=width // 64, dim=64), left_scale=0.8, right_scale=0.9)
+                        rot=dict(dims=dim // 2, base=1e4, scaling=dict(factor=8.0, original=4096, fast=16.0, slow=2.0)))
+            mixer = dict(left=left, right=dict(heads=width // 64, dim=64), left_scale=0.7, right_scale=1.2)
             listed.append(dict(type="parallel", mixer=mixer, mlp=dict(kind="dense", ff=ff)))
         else:
             mixer = dict(heads=heads, kv_heads=kv, dim=dim, vdim=dim, scale=dim ** -0.5, v_mix=True,
-                         rot=dict(dims=dim // 2, base=5e5), mask=dict(size=DESIGN_WINDOW, keep_first=DESIGN_KEEP))
+                         rot=dict(dims=dim // 2, base=1e4), mask=dict(size=DESIGN_WINDOW, keep_first=DESIGN_KEEP))
             listed.append(dict(type="attention", mixer=mixer, mlp=dict(kind="dense", ff=ff)))
     return lab.NinisunConfig.from_dict(dict(architecture="Ninisun", vocab=DESIGN_VOCAB, width=width,
                                             norm=dict(eps=1e-6), layers=listed))

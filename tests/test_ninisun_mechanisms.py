@@ -75,7 +75,7 @@ def test_gelu_gate_as_the_epilogue_of_a_product(backend, dtype, rows):
 
 # ------------------------------------------------------------------ rotation
 @pytest.mark.parametrize("rotation", [
-    dict(dims=8, base=10000.0), dict(dims=24, base=1e6, scaling=dict(factor=4.0, original=1024, fast=32.0, slow=1.0)),
+    dict(dims=8, base=10000.0), dict(dims=20, base=2e5, scaling=dict(factor=3.0, original=512, fast=16.0, slow=2.0)),
     dict(dims=16, base=500.0, scaling=dict(factor=8.0, original=64, fast=4.0, slow=0.5)),
     dict(dims=2, base=7.0, scaling=dict(factor=2.0, original=16, fast=2.0, slow=2.0)),
 ])
@@ -195,6 +195,8 @@ def test_sigmoid_weights_over_prompts_and_decoded_rows(backend, dtype, H_, G, D,
     """No softmax: every visible key weighs sigmoid(score + bias of the head), nothing is
     normalised.  Portions of prompts behind a history, tiles of rows that hold two requests, single
     decoded rows behind hundreds of keys (cut into shares and merged), the very first position."""
+    if backend == "emu" and H_ * (D + E) > 1400:
+        pytest.skip("the references on the CPU take the small shapes; the kernels all of them")
     ops = ops_of(backend)
     lengths, new = [330, 45, 70, 1, 150], [50, 45, 1, 1, 1]
     stand = [(0, 329, 3), (0, 300, 299), (1, 44, 0), (2, 69, 17), (4, 149, 64)]      # far keys, page borders
@@ -218,10 +220,12 @@ def test_sigmoid_weights_over_prompts_and_decoded_rows(backend, dtype, H_, G, D,
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H_,G,D,E", [(4, 2, 16, 24), (4, 2, 32, 16), (8, 2, 64, 32), (8, 2, 96, 192), (2, 1, 128, 256)])
-@pytest.mark.parametrize("window,keep_first", [(24, 3), (16, 0), (5, 9), (40, 6), (300, 2)])
+@pytest.mark.parametrize("window,keep_first", [(24, 3), (16, 0), (5, 9), (48, 7), (300, 2)])
 def test_softmax_without_a_sink_at_the_window_s_edges(backend, dtype, H_, G, D, E, window, keep_first):
     """The plain softmax (no sink) through a window with a kept prefix: a key that would take nearly
     all the weight sits just inside or just outside, in a prompt's portion and for a decoded row."""
+    if backend == "emu" and H_ * (D + E) > 1400:
+        pytest.skip("the references on the CPU take the small shapes; the kernels all of them")
     ops = ops_of(backend)
     for decode in (False, True):
         n = 130
