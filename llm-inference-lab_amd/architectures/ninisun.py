@@ -4,7 +4,7 @@ A stack of layers with a norm before and behind each sublayer and a learned scal
 normed result: ``x += ls1 * norm1b(mixer(norm1(x)))``, then (where the layer has one) ``x +=
 ls2 * norm2b(feed_forward(norm2(x)))``, all RMS norms.  The mixer is grouped-query attention
 (neighbouring channels turned by position, a sliding window that keeps the first positions,
-values mixed with the first such layer's), or two mixers side by side: attention with sigmoid
+values mixed with the first such layer's), or a pair of mixers on one input: attention with sigmoid
 weights and a gate per head, and a recurrent state under a generalised delta rule.  The
 feed-forward is gated with the tanh form of gelu.  The head is the embedding table behind a
 last norm.

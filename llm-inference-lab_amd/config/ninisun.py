@@ -4,7 +4,7 @@ The file lists the layers one by one: each has a ``type`` (which mixer it has), 
 and constants (``mixer``), and its feed-forward (``mlp``, or null for a layer with the mixer
 only).  ``attention``: grouped-query attention with a rotation of neighbouring channels, a
 sliding window that keeps a sequence's first positions, and values that may be mixed with those
-of the first such layer.  ``parallel``: two mixers side by side, a ``left`` one (attention with
+of the first such layer.  ``parallel``: a pair of mixers on one input, a ``left`` one (attention with
 sigmoid weights, biases, a rotation with stretched frequencies and a gate per head) and a
 ``right`` one (a recurrent state under a generalised delta rule), summed with two fixed weights.
 Sizes that the file does not name (the rank of the decay projection) are read off the tensors'

@@ -247,7 +247,8 @@ template <typename T>
 __global__ __launch_bounds__(1024) void gla_output_kernel(const float* __restrict__ parts, int slices, int n_heads, int E,
                                                           const float* __restrict__ w, float eps,
                                                           const float* __restrict__ proj, int ld, int off_g,
-                                                          T* __restrict__ out, int w_per_head, int gate_kind) {
+                                                          T* __restrict__ out, int w_per_head, int gate_kind,
+                                                          int count) {
   __shared__ float red[17];
   const int r = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
   float o = 0.f;
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(1024) void gla_output_kernel(const float* __restric
     const float* p = parts + (((size_t)r * n_heads + h) * slices) * E + e;
     for (int s = 0; s < slices; ++s) o += p[(size_t)s * E];
   }
-  const float ms = block_sum(o * o, red) / (float)E;
+  const float ms = block_sum(o * o, red) / (float)count;      // (count < E: the channels behind it are zeros)
   if (e < E) {
     const float g = proj[(size_t)r * ld + off_g + h * E + e];
     const float y = o * (1.0f / sqrtf(ms + eps)) * w[w_per_head ? h * E + e : e];
@@ -264,22 +265,25 @@ __global__ __launch_bounds__(1024) void gla_output_kernel(const float* __restric
   }
 }
 
-// slices > 0: that many pieces per output (0: as the gated scan leaves them, one per SLICE key channels)
+// slices > 0: that many pieces per output (0: as the gated scan leaves them, one per SLICE key channels);
+// norm_count > 0: the mean of the squares is taken over so many channels (the others are zeros)
 extern "C" int llmlab_gla_output(const float* parts, int rows, int n_heads, int D, int E, const float* w, float eps,
                                  const float* proj, int ld, int off_g, void* out, int dtype, int slices_given,
-                                 int w_per_head, int gate_kind, hipStream_t stream) {
+                                 int w_per_head, int gate_kind, int norm_count, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && n_heads > 0 && n_heads <= 65535 && E > 0 && E <= 1024,
                  "gla_output: bad sizes rows=%d heads=%d E=%d", rows, n_heads, E);
   LLMLAB_REQUIRE(gate_kind == 0 || gate_kind == 1, "gla_output: unknown gate %d", gate_kind);
+  LLMLAB_REQUIRE(norm_count >= 0 && norm_count <= E, "gla_output: a mean over %d of %d channels", norm_count, E);
+  const int count = norm_count > 0 ? norm_count : E;
   if (rows == 0) return 0;
   const int slices = slices_given > 0 ? slices_given : (D + SLICE - 1) / SLICE;
   dim3 grid(rows, n_heads), block((E + 63) / 64 * 64);
   if (dtype == DT_BF16)
     hipLaunchKernelGGL(gla_output_kernel<bf16_t>, grid, block, 0, stream, parts, slices, n_heads, E, w, eps, proj, ld,
-                       off_g, (bf16_t*)out, w_per_head, gate_kind);
+                       off_g, (bf16_t*)out, w_per_head, gate_kind, count);
   else
     hipLaunchKernelGGL(gla_output_kernel<float>, grid, block, 0, stream, parts, slices, n_heads, E, w, eps, proj, ld,
-                       off_g, (float*)out, w_per_head, gate_kind);
+                       off_g, (float*)out, w_per_head, gate_kind, count);
   LLMLAB_LAUNCH_CHECK("gla_output");
   return 0;
 }
@@ -289,7 +293,7 @@ extern "C" int llmlab_gla_output(const float* parts, int rows, int n_heads, int 
 // A matrix-valued state per head whose transition is a decay per key channel less a rank-one
 // removal along the unit key, before the new key/value pair is written:
 //   u_t = k_t / sqrt(|k_t|^2 + key_eps)
-//   S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T        (both terms read S_(t-1))
+//   S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T        (decay and removal act on S_(t-1))
 //   o_t = S_t^T r_t
 // with w_t (decay) and a_t (removal rate) in (0, 1) per head and key channel.  State [D, E]
 // per head, float32, one slot per request; everything here is float32.

@@ -1114,7 +1114,7 @@ class HipOps:
                                                 _c_ptr, _c_int, _c_ptr]
                 lib.llmlab_gla_scan.restype = _c_int
                 lib.llmlab_gla_output.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_float, _c_ptr,
-                                                  _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
+                                                  _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr]
                 lib.llmlab_gla_output.restype = _c_int
                 lib.llmlab_delta_gates.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
                                                    _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
@@ -1574,11 +1574,13 @@ class HipOps:
 
     OUTPUT_GATES = {"silu": 0, "sigmoid": 1}
 
-    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out, gate: str = "silu") -> None:
+    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out, gate: str = "silu",
+                   norm_count: int = 0) -> None:
         """``out[r, h] = rmsnorm(sum of parts[r, h]) * weight * silu(gate[r, h])`` with the gate at
         column ``off_gate`` of the float32 ``proj``; ``out`` in the compute dtype.  ``parts [rows, heads,
         pieces, value_dim]`` with any number of pieces; ``weight`` of ``value_dim`` numbers (the same for
-        every head) or of ``heads * value_dim``; ``gate="sigmoid"``: ``... * sigmoid(gate[r, h])``."""
+        every head) or of ``heads * value_dim``; ``gate="sigmoid"``: ``... * sigmoid(gate[r, h])``; ``norm_count``:
+        the mean of the squares is taken over so many channels of a head (the ones behind them are zeros)."""
         lib = self._mixer_lib("linear_attention")
         self._need(parts, "output pieces", torch.float32)
         self._need(proj, "projections", torch.float32)
@@ -1593,7 +1595,7 @@ class HipOps:
         per_head = 1 if weight.numel() == num_heads * value_dim and num_heads > 1 else 0
         self._call(lib.llmlab_gla_output, self._ptr(parts), rows, num_heads, key_dim, value_dim, self._ptr(weight),
                    float(eps), self._ptr(proj), proj.stride(0), int(off_gate), self._ptr(out), _dt(out),
-                   int(parts.shape[2]), per_head, self.OUTPUT_GATES[gate], self._stream(), lib=lib)
+                   int(parts.shape[2]), per_head, self.OUTPUT_GATES[gate], int(norm_count or 0), self._stream(), lib=lib)
 
     def delta_gates(self, proj, off_low, rank, off_rate, off_k, w2, w0, rate_bias, decay_scale, key_eps, num_heads,
                     key_dim, decay, unit, removal) -> None:

@@ -321,7 +321,10 @@ class WindowedSinkAttention(Mixer):
     ``(1 - lambda) v + lambda v_first`` with ``v_first`` what the ``"first"`` layer left for the same
     token and ``lambda`` one learned number (role ``value_mix``); the mixed values are what is cached.
 
-    Pages: keys ``[kv_heads, P, key_dim]``, values ``[kv_heads, P, value_dim]``."""
+    Pages: keys ``[kv_heads, P, key_dim]``, values ``[kv_heads, P, value_dim]``.  The products'
+    inner sizes are multiples of 8: a value head of another width is laid out with zeros behind
+    its channels (zero rows of the value projection, zero columns of the output projection), which
+    changes no output."""
 
     writes_output = True
     takes_normed_input = True      # (few rows: the norm in front of the mixer runs inside its first product)
@@ -361,7 +364,9 @@ class WindowedSinkAttention(Mixer):
         self.b_in = self.score_bias = None
         self.mix_weight = 0.0
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
-        self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.key_dim = int(key_dim)
+        self.file_value_dim = int(value_dim)                       # a value head as the model file has it
+        self.value_dim = (self.file_value_dim + 7) // 8 * 8        # and as the kernels and the pages see it
         self.scale = float(scale)
         self.window = None if window is None else int(window)
         self.keep_first = int(keep_first or 0)
@@ -387,15 +392,16 @@ class WindowedSinkAttention(Mixer):
 
     def tensor_specs(self):
         t, w = self.tensor_names, self.hidden_size
+        file_v = self.num_kv_heads * self.file_value_dim
         specs = {t["q_weight"]: TensorSpec((self.q_size, w), MATRIX),
-                 t["o_weight"]: TensorSpec((w, self.num_heads * self.value_dim), MATRIX)}
+                 t["o_weight"]: TensorSpec((w, self.num_heads * self.file_value_dim), MATRIX)}
         if self.own_kv:
             specs[t["k_weight"]] = TensorSpec((self.k_size, w), MATRIX)
-            specs[t["v_weight"]] = TensorSpec((self.v_size, w), MATRIX)
+            specs[t["v_weight"]] = TensorSpec((file_v, w), MATRIX)
         if self.qkv_bias:
             specs[t["q_bias"]] = TensorSpec((self.q_size,), VECTOR)
             specs[t["k_bias"]] = TensorSpec((self.k_size,), VECTOR)
-            specs[t["v_bias"]] = TensorSpec((self.v_size,), VECTOR)
+            specs[t["v_bias"]] = TensorSpec((file_v,), VECTOR)
         if self.has_score_bias:
             specs[t["score_bias"]] = TensorSpec((self.num_heads,), VECTOR)
         if self.output_gate:
@@ -418,14 +424,24 @@ class WindowedSinkAttention(Mixer):
         ops.check_product_sizes(self.hidden_size, dtype, "attention projections (hidden size)")
         ops.check_product_sizes(self.num_heads * self.value_dim, dtype, "attention output projection (heads * value size)")
         t = self.tensor_names
+        e, ek = self.file_value_dim, self.value_dim
+
+        def value_heads(x, heads):
+            """Rows (or entries) of ``heads`` value heads of ``e`` channels -> of ``ek``, zeros behind."""
+            if e == ek:
+                return x
+            per_head = x.unflatten(0, (heads, e))
+            zeros = torch.zeros((heads, ek - e) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+            return torch.cat([per_head, zeros], dim=1).flatten(0, 1)
         rows = [tensors[t["q_weight"]]]
         if self.own_kv:
-            rows += [tensors[t["k_weight"]], tensors[t["v_weight"]]]
+            rows += [tensors[t["k_weight"]], value_heads(tensors[t["v_weight"]], self.num_kv_heads)]
         if self.output_gate:
             rows.append(tensors[t["gate_weight"]])
         self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())       # one product for q (, k, v, gates)
         if self.qkv_bias:
-            bias = [tensors[t[r]].float() for r in ("q_bias", "k_bias", "v_bias")]
+            bias = [tensors[t["q_bias"]].float(), tensors[t["k_bias"]].float(),
+                    value_heads(tensors[t["v_bias"]].float(), self.num_kv_heads)]
             if self.output_gate:
                 bias.append(torch.zeros(self.num_heads, dtype=torch.float32, device=bias[0].device))
             self.b_in = torch.cat(bias).contiguous()
@@ -435,7 +451,7 @@ class WindowedSinkAttention(Mixer):
             self.mix_weight = float(tensors[t["value_mix"]].float().reshape(-1)[0])
         if self.position is not None:
             self.position.bind(tensors, ops, dtype)
-        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
+        self.w_o = ops.prepare_weight(value_heads(tensors[t["o_weight"]].t(), self.num_heads).t().contiguous())
         if self.qk_norm:
             self.q_norm = tensors[t["q_norm"]].float().contiguous()
             self.k_norm = tensors[t["k_norm"]].float().contiguous() if self.own_kv else None

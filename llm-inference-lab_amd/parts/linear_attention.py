@@ -160,8 +160,8 @@ class DeltaRuleAttention(Mixer):
     and removal rates ``a = sigmoid(Wa h + ba)``, both per head and key channel; per head, token by
     token, with the unit key ``u = k / sqrt(|k|^2 + key_eps)``::
 
-        S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T     (S is D x E; both terms
-        o_t = S_t^T r_t                                                        read the old state)
+        S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T     (S is D x E; decay and removal
+        o_t = S_t^T r_t                                                        both act on S_(t-1))
 
     then every head's ``o_t`` is divided by its root mean square over ``E`` (``norm_eps`` inside the
     root), the heads are put side by side, multiplied by a weight of all heads' size and by
@@ -187,7 +187,9 @@ class DeltaRuleAttention(Mixer):
                  gate: str = "sigmoid"):
         super().__init__(tensors)
         self.hidden_size, self.num_heads, self.key_dim = int(hidden_size), int(num_heads), int(key_dim)
-        self.value_dim = self.key_dim if value_dim is None else int(value_dim)
+        self.file_value_dim = self.key_dim if value_dim is None else int(value_dim)      # as the model file has it
+        # (the products' inner sizes are multiples of 8: zeros behind a head's value channels)
+        self.value_dim = (self.file_value_dim + 7) // 8 * 8
         self.decay_rank = None if decay_rank is None else int(decay_rank)
         self.decay_scale, self.key_eps, self.norm_eps = float(decay_scale), float(key_eps), float(norm_eps)
         if gate not in ("sigmoid", "silu"):
@@ -207,18 +209,19 @@ class DeltaRuleAttention(Mixer):
 
     def tensor_specs(self):
         t, w = self.tensor_names, self.hidden_size
+        file_v = self.num_heads * self.file_value_dim
         return {
             t["r_weight"]: TensorSpec((self.qk_size, w), MATRIX),
             t["k_weight"]: TensorSpec((self.qk_size, w), MATRIX),
-            t["v_weight"]: TensorSpec((self.v_size, w), MATRIX),
-            t["gate_weight"]: TensorSpec((self.v_size, w), MATRIX),
+            t["v_weight"]: TensorSpec((file_v, w), MATRIX),
+            t["gate_weight"]: TensorSpec((file_v, w), MATRIX),
             t["rate_weight"]: TensorSpec((self.qk_size, w), MATRIX),
             t["rate_bias"]: TensorSpec((self.qk_size,), VECTOR),
             t["decay_down"]: TensorSpec((self.decay_rank, w), MATRIX),
             t["decay_up"]: TensorSpec((self.qk_size, self.decay_rank), MATRIX),
             t["decay_bias"]: TensorSpec((self.qk_size,), VECTOR),
-            t["out_norm"]: TensorSpec((self.v_size,), VECTOR, INIT_NORM),
-            t["o_weight"]: TensorSpec((w, self.v_size), MATRIX),
+            t["out_norm"]: TensorSpec((file_v,), VECTOR, INIT_NORM),
+            t["o_weight"]: TensorSpec((w, file_v), MATRIX),
         }
 
     def bind(self, tensors, ops, dtype):
@@ -233,20 +236,29 @@ class DeltaRuleAttention(Mixer):
                              f"{int(tensors[t['decay_up']].shape[1])} columns: the two factors of the decay "
                              f"projection do not fit")
         self.decay_rank = rank
+        e, ek = self.file_value_dim, self.value_dim
+
+        def value_heads(x):
+            """Rows (or entries) of the heads' ``e`` value channels -> of ``ek``, zeros behind."""
+            if e == ek:
+                return x
+            per_head = x.unflatten(0, (self.num_heads, e))
+            zeros = torch.zeros((self.num_heads, ek - e) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+            return torch.cat([per_head, zeros], dim=1).flatten(0, 1)
         # one product for r, k, v, the gate, the rates and the low-rank input of the decays
         self.offsets, at, rows = {}, 0, []
         for role in ("r_weight", "k_weight", "v_weight", "gate_weight", "rate_weight", "decay_down"):
             self.offsets[role] = at
-            rows.append(tensors[t[role]])
+            rows.append(value_heads(tensors[t[role]]) if role in ("v_weight", "gate_weight") else tensors[t[role]])
             at += rows[-1].shape[0]
         self.in_size = at
         self.w_in = ops.prepare_weight(torch.cat(rows, dim=0).contiguous())
-        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
+        self.w_o = ops.prepare_weight(value_heads(tensors[t["o_weight"]].t()).t().contiguous())
         # the second factor of the decays is applied in float32, inside the gates' kernel
         self.w_decay = tensors[t["decay_up"]].float().contiguous()
         self.b_decay = tensors[t["decay_bias"]].float().contiguous()
         self.b_rate = tensors[t["rate_bias"]].float().contiguous()
-        self.norm_weight = tensors[t["out_norm"]].float().contiguous()
+        self.norm_weight = value_heads(tensors[t["out_norm"]].float()).contiguous()
 
     def _min_chunk(self) -> int:
         rules = getattr(self.ops, "rules", None)
@@ -288,8 +300,12 @@ class DeltaRuleAttention(Mixer):
         else:
             scan()
         mixed = ctx.scratch("delta_rule.out", (rows, self.v_size), self.dtype)
-        ops.gla_output(outs, self.num_heads, self.key_dim, self.value_dim, self.norm_weight, self.norm_eps, proj,
-                       o["gate_weight"], mixed, self.gate)
+        if self.file_value_dim != self.value_dim:      # (the heads' unit norm is over the file's channels)
+            ops.gla_output(outs, self.num_heads, self.key_dim, self.value_dim, self.norm_weight, self.norm_eps, proj,
+                           o["gate_weight"], mixed, self.gate, self.file_value_dim)
+        else:
+            ops.gla_output(outs, self.num_heads, self.key_dim, self.value_dim, self.norm_weight, self.norm_eps, proj,
+                           o["gate_weight"], mixed, self.gate)
         ops.linear_logits(mixed, self.w_o, out)
 
     def forward(self, h, residual, ctx, entry):

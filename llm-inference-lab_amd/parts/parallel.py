@@ -1,4 +1,4 @@
-"""Two mixers side by side."""
+"""A mixer made of two: both on one input, their results summed."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -25,7 +25,7 @@ class ParallelMixers(Mixer):
         self.left, self.right = build_part("mixer", left), build_part("mixer", right)
         self.left_scale, self.right_scale = float(left_scale), float(right_scale)
         if self.left.cache_spec() is not None and self.right.cache_spec() is not None:
-            raise ValueError("two mixers side by side share one run of the schedule: only one of them may keep a cache")
+            raise ValueError("the two mixers share one run of the schedule: only one of them may keep a cache")
         clash = set(self.left.state_spec()) & set(self.right.state_spec())
         if clash:
             raise ValueError(f"both mixers keep per-request state called {sorted(clash)}")

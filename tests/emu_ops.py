@@ -441,11 +441,12 @@ class EmuOps:
                 for s in range(parts.shape[2]):
                     parts[t, :, s] = o[:, s * S:(s + 1) * S].sum(1)
 
-    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out, gate="silu"):
+    def gla_output(self, parts, num_heads, key_dim, value_dim, weight, eps, proj, off_gate, out, gate="silu",
+                   norm_count=0):
         self._count("gla_output")
         o = parts.sum(2)                                        # [rows, H, E]
         w = weight.float().view(num_heads, value_dim) if weight.numel() == num_heads * value_dim else weight.float()
-        y = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * w
+        y = o / torch.sqrt((o * o).sum(-1, keepdim=True) / (norm_count or value_dim) + eps) * w
         g = proj[:, off_gate:off_gate + num_heads * value_dim].float().view(-1, num_heads, value_dim)
         out.copy_((y * (g if gate == "silu" else 1.0) * torch.sigmoid(g)).reshape(out.shape).to(out.dtype))
 

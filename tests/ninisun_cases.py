@@ -44,6 +44,8 @@ def parallel(left, right, left_scale, right_scale, ff=None):
 # Q: parallel layers only with one key/value head, a state wider than 32, weights far from 1.
 # R: attention only: kv_heads == heads, a kept prefix longer than the window, one layer without a
 #    mask, a window longer than any test sequence, a single mixing layer.
+# S: sizes that are multiples of 2 or 4 and nothing more: heads times value width (36, 60) and the
+#    state's width (36) are no multiples of 8, a feed-forward of 52, a key head of 10 channels.
 CONFIGS = {
     "P": dict(architecture="Ninisun", vocab=211, width=64, norm=dict(eps=1e-5), layers=[
         parallel((4, 2, 16, 32, 0.9, rot(8, 10000.0, (8.0, 64, 4.0, 0.5))), (3, 16), 0.7, 1.3, ff=96),
@@ -55,6 +57,11 @@ CONFIGS = {
     "Q": dict(architecture="Ninisun", vocab=97, width=48, norm=dict(eps=1e-6), layers=[
         parallel((2, 1, 24, 8, 1.2, rot(24, 50.0, (2.0, 16, 2.0, 1.0))), (1, 40), 1.9, 0.2),
         parallel((3, 1, 8, 40, 2.0, rot(2, 7.0)), (2, 24), 0.3, 1.1, ff=56),
+    ]),
+    "S": dict(architecture="Ninisun", vocab=77, width=40, norm=dict(eps=1e-5), layers=[
+        attention(3, 3, 10, 12, 0.7, rot(6, 100.0), size=13, keep_first=2, v_mix=True, ff=52),
+        parallel((3, 1, 12, 20, 0.6, rot(4, 1000.0, (2.0, 32, 4.0, 1.0))), (3, 12), 0.9, 1.4, ff=52),
+        attention(6, 3, 14, 12, 0.5, rot(14, 20.0), size=30, keep_first=0, v_mix=True),
     ]),
     "R": dict(architecture="Ninisun", vocab=130, width=72, norm=dict(eps=1e-6), layers=[
         attention(3, 3, 24, 72, 1.2, rot(6, 2000.0), size=7, keep_first=9, ff=40),

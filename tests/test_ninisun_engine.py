@@ -10,7 +10,7 @@ import plain_ninisun
 from emu_ops import EmuOps
 
 BACKENDS = ["emu", pytest.param("hip", marks=pytest.mark.gpu)]
-LENGTHS = {"P": [1, 9, 37, 83], "Q": [2, 30, 71], "R": [5, 52, 90]}
+LENGTHS = {"P": [1, 9, 37, 83], "Q": [2, 30, 71], "R": [5, 52, 90], "S": [4, 41, 66]}
 # Logits have a standard deviation of about 2.  float32: sums in another order than the float64
 # plain implementation.  bfloat16: bounds on the root mean square and the largest difference over
 # all logits, twice what the kernels' references in float32 arithmetic with the same roundings
@@ -45,7 +45,7 @@ CUTS = {"whole": H.steps_whole, "decode": H.steps_prefill_then_decode, "token by
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 @pytest.mark.parametrize("cut", list(CUTS))
 def test_every_cut_matches_plain(backend, name, cut):
     """Whole prompts, decoding, portions down to two tokens, mixed batches with few pages and
@@ -63,7 +63,7 @@ def test_every_cut_matches_plain(backend, name, cut):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_bfloat16_mixed_batches(backend, name):
     seqs = sequences_of(name)
     want = {rid: N.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
